@@ -38,14 +38,14 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
 
 // embedding rows of any width (the shared gather moves four elements at a time)
 __global__ __launch_bounds__(256) void lay_embed_rows_kernel(const uint16_t* __restrict__ emb, const uint32_t* __restrict__ ids,
-                                                             float* __restrict__ x, int W, int V) {
+                                                             float* __restrict__ x, int W, int V, float scale) {
     uint32_t tok = ids[blockIdx.x];
     if (tok >= (uint32_t)V) tok = 0;
-    for (int i = threadIdx.x; i < W; i += 256) x[(size_t)blockIdx.x * W + i] = bf16_to_f32(emb[(size_t)tok * W + i]);
+    for (int i = threadIdx.x; i < W; i += 256) x[(size_t)blockIdx.x * W + i] = bf16_to_f32(emb[(size_t)tok * W + i]) * scale;
 }
-void launch_lay_embed_rows(const uint16_t* emb, const uint32_t* ids, float* x, int T, int W, int V, hipStream_t s) {
+void launch_lay_embed_rows(const uint16_t* emb, const uint32_t* ids, float* x, int T, int W, int V, hipStream_t s, float scale) {
     if (T <= 0) return;
-    hipLaunchKernelGGL(lay_embed_rows_kernel, dim3((unsigned)T), dim3(256), 0, s, emb, ids, x, W, V);
+    hipLaunchKernelGGL(lay_embed_rows_kernel, dim3((unsigned)T), dim3(256), 0, s, emb, ids, x, W, V, scale);
 }
 
 // ------------------------------------------------------------------------------------------------------------------
@@ -152,11 +152,28 @@ void launch_lay_add_norm2_shift_decode(float* x, const float* y1, const float* y
 // rotation by position: the angle and its sine / cosine are f32 (sincosf reduces the argument exactly)
 __global__ __launch_bounds__(256) void lay_rope_kernel(const float* src, int lds, int s_vstride, float* dst, int ldd, int d_vstride, int nvec,
                                                        int len, int dims, const float* __restrict__ freq, float mag,
-                                                       const LaySegDev* __restrict__ segs, const int32_t* __restrict__ rowseg) {
+                                                       const LaySegDev* __restrict__ segs, const int32_t* __restrict__ rowseg, int half) {
     const int r = blockIdx.x;
     const LaySegDev sg = segs[rowseg[r]];
     const float pos = (float)(sg.start_pos + (r - sg.row0));
     const int hp = (len + 1) / 2;
+    if (half) {                            // pairs (i, i + dims / 2); a thread owns both elements of its pair, so dst may be src
+        const int hd = dims / 2, per = hd + (len - dims);
+        for (int idx = threadIdx.x; idx < nvec * per; idx += 256) {
+            const int v = idx / per, i = idx - v * per;
+            const float* sp = src + (size_t)r * lds + (size_t)v * s_vstride;
+            float* dp = dst + (size_t)r * ldd + (size_t)v * d_vstride;
+            if (i < hd) {
+                const float a = sp[i], b = sp[i + hd];
+                float sn, cs;
+                sincosf(pos * freq[i], &sn, &cs);
+                sn *= mag; cs *= mag;
+                dp[i] = a * cs - b * sn;
+                dp[i + hd] = b * cs + a * sn;
+            } else dp[dims + (i - hd)] = sp[dims + (i - hd)];
+        }
+        return;
+    }
     for (int idx = threadIdx.x; idx < nvec * hp; idx += 256) {
         const int v = idx / hp, i = idx - v * hp;
         const float* sp = src + (size_t)r * lds + (size_t)v * s_vstride + 2 * i;
@@ -176,10 +193,10 @@ __global__ __launch_bounds__(256) void lay_rope_kernel(const float* src, int lds
     }
 }
 void launch_lay_rope(const float* src, int lds, int s_vstride, float* dst, int ldd, int d_vstride, int nvec, int len, int dims,
-                     const float* freq, float mag, const LaySegDev* segs, const int32_t* rowseg, int T, hipStream_t s) {
+                     const float* freq, float mag, const LaySegDev* segs, const int32_t* rowseg, int T, hipStream_t s, bool half) {
     if (T <= 0 || nvec <= 0 || len <= 0) return;
     hipLaunchKernelGGL(lay_rope_kernel, dim3((unsigned)T), dim3(256), 0, s, src, lds, s_vstride, dst, ldd, d_vstride, nvec, len, dims, freq, mag,
-                       segs, rowseg);
+                       segs, rowseg, half ? 1 : 0);
 }
 
 __global__ __launch_bounds__(256) void lay_rms_gate_kernel(const float* __restrict__ o, const float* __restrict__ gate, int ldg,
@@ -802,6 +819,59 @@ void launch_lay_k_append(const float* proj, int ldp, int k_off, void* kpool, int
     else hipLaunchKernelGGL(lay_k_append_kernel<KV_BF16>, dim3((unsigned)T), dim3(256), 0, s, proj, ldp, k_off, kpool, bt, segs, rowseg, G, d, page);
 }
 
+// the cached row behind entry v of a tile's key walk: [0, front) are the kept first tokens or -- pool > 0 -- the mean rows of the
+// position blocks (block v lives in the page of its last position), then the window from main_lo on
+struct LaRow { const char* k; const char* v; };
+template <int ESZ>
+__device__ __forceinline__ LaRow la_row(const LAttnArgs& a, const LaySegDev& sg, int g, int v, int front, int main_lo, int pool) {
+    LaRow r;
+    if (pool > 0 && v < front) {
+        const int lpg = (v * pool + pool - 1) / a.page;
+        const int idx = v - (int)(((long long)lpg * a.page) / pool);
+        const size_t row = ((size_t)a.bt[sg.bt_off + lpg] * a.G + g) * a.pool_rows + idx;
+        r.k = (const char*)a.pk_pool + row * a.d * ESZ;
+        r.v = a.pv_pool ? (const char*)a.pv_pool + row * a.e * ESZ : nullptr;
+    } else {
+        const int j = v < front ? v : main_lo + (v - front);
+        const size_t row = ((size_t)a.bt[sg.bt_off + j / a.page] * a.G + g) * a.page + (size_t)(j % a.page);
+        r.k = (const char*)a.kpool + row * a.d * ESZ;
+        r.v = a.vpool ? (const char*)a.vpool + row * a.e * ESZ : nullptr;
+    }
+    return r;
+}
+
+// one block per row of the pass; a row whose position closes a block of `pool` positions writes the block's mean row (f32 sum in
+// position order, then one rounding into the cache's format)
+template <int KVT>
+__global__ __launch_bounds__(256) void lay_pool_append_kernel(const void* __restrict__ kpool, void* __restrict__ pk_pool,
+                                                              const int32_t* __restrict__ bt, const LaySegDev* __restrict__ segs,
+                                                              const int32_t* __restrict__ rowseg, int G, int d, int page, int pool, int pool_rows) {
+    const int r = blockIdx.x;
+    const LaySegDev sg = segs[rowseg[r]];
+    const int pos = sg.start_pos + (r - sg.row0);
+    if ((pos + 1) % pool != 0) return;
+    const int b = (pos + 1) / pool - 1, lpg = pos / page;
+    const int idx = b - (int)(((long long)lpg * page) / pool);
+    const float inv = 1.f / (float)pool;
+    for (int i = threadIdx.x; i < G * d; i += 256) {
+        const int g = i / d, c = i - g * d;
+        float sum = 0.f;
+        for (int j = b * pool; j <= pos; ++j) {
+            const size_t src = (((size_t)bt[sg.bt_off + j / page] * G + g) * page + (size_t)(j % page)) * d + c;
+            sum += KVT == KV_F32 ? ((const float*)kpool)[src] : bf16_to_f32(((const uint16_t*)kpool)[src]);
+        }
+        const size_t dst = (((size_t)bt[sg.bt_off + lpg] * G + g) * pool_rows + idx) * d + c;
+        if (KVT == KV_F32) ((float*)pk_pool)[dst] = sum * inv;
+        else ((uint16_t*)pk_pool)[dst] = f32_to_bf16(sum * inv);
+    }
+}
+void launch_lay_pool_append(const void* kpool, void* pk_pool, int kvt, const int32_t* bt, const LaySegDev* segs, const int32_t* rowseg, int T,
+                            int G, int d, int page, int pool, int pool_rows, hipStream_t s) {
+    if (T <= 0 || pool <= 0) return;
+    if (kvt == KV_F32) hipLaunchKernelGGL(lay_pool_append_kernel<KV_F32>, dim3((unsigned)T), dim3(256), 0, s, kpool, pk_pool, bt, segs, rowseg, G, d, page, pool, pool_rows);
+    else hipLaunchKernelGGL(lay_pool_append_kernel<KV_BF16>, dim3((unsigned)T), dim3(256), 0, s, kpool, pk_pool, bt, segs, rowseg, G, d, page, pool, pool_rows);
+}
+
 // A block = 16 query rows of one sequence and one key head: row qi = (position in the portion) * nrep + (query head in the
 // group), so that a single decode token fills the tile with the heads that share its keys.  16 lanes per query row.
 // Keys the tile can see: the kept first tokens [0, min(keep, lo)) and the window [lo, last position], lo not before the start of
@@ -838,14 +908,14 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
     int main_lo = max(0, pmin - win + 1);
     if (chunk > 0) main_lo = max(main_lo, pmin / chunk * chunk);
     const int clo = chunk > 0 ? pos / chunk * chunk : 0;       // first position of this query's block
-    const int sink_hi = min(keep, main_lo);
+    const int pool = (int)min(a.pool, 1ll << 30);
+    const int sink_hi = pool > 0 ? max(0, (pmax - win + 1) / pool) : min(keep, main_lo);
     const int total = sink_hi + (pmax - main_lo + 1);
     const float r1 = a.bias != LBIAS_NONE ? a.r1[head] : 0.f, r2 = a.bias == LBIAS_LOG ? a.r2[head] : 0.f;
     float m = -INFINITY, l = 0.f, acc[NACC];
     if (a.sink && blockIdx.z == 0 && qvalid) { m = a.sink[head]; l = 1.f; }
 #pragma unroll
     for (int c = 0; c < NACC; ++c) acc[c] = 0.f;
-    const size_t esz = KVT == KV_F32 ? 4 : 2;
     const int nsplit = (int)gridDim.z;     // the visible keys' tiles are dealt round-robin to nsplit blocks (few queries, many keys)
     __syncthreads();                       // qs written (a split may have no tile at all)
     for (int v0 = (int)blockIdx.z * KT; v0 < total; v0 += KT * nsplit) {
@@ -854,9 +924,8 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
             const int sl = qr + 16 * rr;
             const int v = v0 + sl;
             if (v < total) {
-                const int j = v < sink_hi ? v : main_lo + (v - sink_hi);
-                const int pg = a.bt[sg.bt_off + j / a.page];
-                const char* src = (const char*)a.kpool + ((((size_t)pg * a.G + g) * a.page + (size_t)(j % a.page)) * d) * esz;
+                const LaRow cr = la_row<(KVT == KV_F32 ? 4 : 2)>(a, sg, g, v, sink_hi, main_lo, pool);
+                const char* src = cr.k;
                 if (KVT != KV_F32 && (d & 7) == 0) {             // 16 bytes = 8 cached keys per lane and load
                     for (int i = ln * 8; i < d; i += 128) {
                         const u32x4 p = *(const u32x4*)((const uint16_t*)src + i);
@@ -868,7 +937,7 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
                 for (int i = ln; i < d; i += 16)
                     ks[sl * ldk + i] = KVT == KV_F32 ? ((const float*)src)[i] : bf16_to_f32(((const uint16_t*)src)[i]);
                 if (ownv) {
-                    const char* vsrc = (const char*)a.vpool + ((((size_t)pg * a.G + g) * a.page + (size_t)(j % a.page)) * e) * esz;
+                    const char* vsrc = cr.v;
                     for (int i = ln; i < e; i += 16)
                         vs[sl * e + i] = KVT == KV_F32 ? ((const float*)vsrc)[i] : bf16_to_f32(((const uint16_t*)vsrc)[i]);
                 }
@@ -888,8 +957,10 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
             float dot = 0.f;
             for (int i = 0; i < d; ++i) dot = fmaf(qs[qr * ldq + i], ks[sl * ldk + i], dot);
             const int dist = pos - j;
-            const bool vis = qvalid && v < total && dist >= 0 && ((dist < win && j >= clo) || j < keep);
-            const float pen = a.bias == LBIAS_LOG ? r1 * log1pf(r2 * (float)dist) : r1 * (float)dist;
+            const bool pl = pool > 0 && v < sink_hi;       // a block's mean row: seen once the whole block lies in front of the window
+            const bool vis = pl ? qvalid && (v + 1) * pool <= pos - win + 1
+                                : qvalid && v < total && dist >= 0 && ((dist < win && j >= clo) || j < keep);
+            const float pen = pl ? 0.f : (a.bias == LBIAS_LOG ? r1 * log1pf(r2 * (float)dist) : r1 * (float)dist);
             sc[c] = vis ? dot * a.scale - pen : -INFINITY;
             tmax = fmaxf(tmax, sc[c]);
         }
@@ -930,7 +1001,7 @@ __global__ __launch_bounds__(256) void lay_attn_kernel(LAttnArgs a) {
     }
     if (!qvalid) return;
     const float* gp = a.proj + (size_t)row * a.ldp + a.g_off + (a.gate == LGATE_ELEM ? head * e : head);
-    const float inv = (a.gate == LGATE_HEAD ? gp[0] : 1.f) / l;
+    const float inv = (a.gate == LGATE_HEAD ? gp[0] : 1.f) / l * a.out_scale;
 #pragma unroll
     for (int c = 0; c < NACC; ++c) {
         const int i = ln + 16 * c;
@@ -993,7 +1064,8 @@ __global__ __launch_bounds__(LM_NT) void lay_attn_mfma_kernel(LAttnArgs a) {
     const int pmin = sg.start_pos + q0 / nrep, pmax = sg.start_pos + (q0 + nq - 1) / nrep;
     int main_lo = max(0, pmin - win + 1);
     if (chunk > 0) main_lo = max(main_lo, pmin / chunk * chunk);
-    const int sink_hi = min(keep, main_lo);
+    const int pool = (int)min(a.pool, 1ll << 30);
+    const int sink_hi = pool > 0 ? max(0, (pmax - win + 1) / pool) : min(keep, main_lo);
     const int total = sink_hi + (pmax - main_lo + 1);
     f32x4 O[NEMAX];
 #pragma unroll
@@ -1012,11 +1084,7 @@ __global__ __launch_bounds__(LM_NT) void lay_attn_mfma_kernel(LAttnArgs a) {
             const int sl = idx / (d / 8), i = (idx - sl * (d / 8)) * 8;
             const int v = v0 + sl;
             u32x4 pk = {0u, 0u, 0u, 0u};
-            if (v < total) {
-                const int j = v < sink_hi ? v : main_lo + (v - sink_hi);
-                const int pg = a.bt[sg.bt_off + j / a.page];
-                pk = *(const u32x4*)((const uint16_t*)a.kpool + (((size_t)pg * a.G + g) * a.page + (size_t)(j % a.page)) * d + i);
-            }
+            if (v < total) pk = *(const u32x4*)((const uint16_t*)la_row<2>(a, sg, g, v, sink_hi, main_lo, pool).k + i);
             *(u32x4*)&Ks[sl * ldq + i] = pk;
             if (!WIDE && !ownv && i < e) {
                 Kt[(i + 0) * ldp + sl] = (uint16_t)(pk.x & 0xFFFFu); Kt[(i + 1) * ldp + sl] = (uint16_t)(pk.x >> 16);
@@ -1030,11 +1098,7 @@ __global__ __launch_bounds__(LM_NT) void lay_attn_mfma_kernel(LAttnArgs a) {
                 const int sl = idx / (e / 8), i = (idx - sl * (e / 8)) * 8;
                 const int v = v0 + sl;
                 u32x4 pk = {0u, 0u, 0u, 0u};
-                if (v < total) {
-                    const int j = v < sink_hi ? v : main_lo + (v - sink_hi);
-                    const int pg = a.bt[sg.bt_off + j / a.page];
-                    pk = *(const u32x4*)((const uint16_t*)a.vpool + (((size_t)pg * a.G + g) * a.page + (size_t)(j % a.page)) * e + i);
-                }
+                if (v < total) pk = *(const u32x4*)((const uint16_t*)la_row<2>(a, sg, g, v, sink_hi, main_lo, pool).v + i);
                 Kt[(i + 0) * ldp + sl] = (uint16_t)(pk.x & 0xFFFFu); Kt[(i + 1) * ldp + sl] = (uint16_t)(pk.x >> 16);
                 Kt[(i + 2) * ldp + sl] = (uint16_t)(pk.y & 0xFFFFu); Kt[(i + 3) * ldp + sl] = (uint16_t)(pk.y >> 16);
                 Kt[(i + 4) * ldp + sl] = (uint16_t)(pk.z & 0xFFFFu); Kt[(i + 5) * ldp + sl] = (uint16_t)(pk.z >> 16);
@@ -1064,8 +1128,10 @@ __global__ __launch_bounds__(LM_NT) void lay_attn_mfma_kernel(LAttnArgs a) {
                 const int v = v0 + t * 16 + lr;
                 const int j = v < sink_hi ? v : main_lo + (v - sink_hi);
                 const int dist = qpos[r] - j;
-                const bool vis = qok[r] && v < total && dist >= 0 && ((dist < win && j >= qclo[r]) || j < keep);
-                const float pen = a.bias == LBIAS_LOG ? r1[r] * __logf(1.f + r2[r] * (float)dist) : r1[r] * (float)dist;
+                const bool pl = pool > 0 && v < sink_hi;
+                const bool vis = pl ? qok[r] && (v + 1) * pool <= qpos[r] - win + 1
+                                    : qok[r] && v < total && dist >= 0 && ((dist < win && j >= qclo[r]) || j < keep);
+                const float pen = pl ? 0.f : (a.bias == LBIAS_LOG ? r1[r] * __logf(1.f + r2[r] * (float)dist) : r1[r] * (float)dist);
                 sc[t] = vis ? S[t][r] * a.scale - pen : -INFINITY;
                 tmax = fmaxf(tmax, sc[t]);
             }
@@ -1112,7 +1178,7 @@ __global__ __launch_bounds__(LM_NT) void lay_attn_mfma_kernel(LAttnArgs a) {
     for (int r = 0; r < 4; ++r) {
         if (!qok[r]) continue;
         const float* gp = a.proj + (size_t)qrow[r] * a.ldp + a.g_off + (a.gate == LGATE_ELEM ? qhead[r] * e : qhead[r]);
-        const float inv = (a.gate == LGATE_HEAD ? gp[0] : 1.f) / l[r];
+        const float inv = (a.gate == LGATE_HEAD ? gp[0] : 1.f) / l[r] * a.out_scale;
 #pragma unroll
         for (int n = 0; n < NEMAX; ++n)
             if (n < ne) a.out[(size_t)qrow[r] * a.ldo + qhead[r] * e + n * 16 + lr] = O[n][r] * inv * (a.gate == LGATE_ELEM ? gp[n * 16 + lr] : 1.f);
@@ -1173,7 +1239,7 @@ __global__ __launch_bounds__(256) void lay_attn_merge_kernel(LAttnArgs a, int ns
             acc = fmaf(a.part_o[pr * d + i], w, acc);
         }
         const float gate = a.gate == LGATE_NONE ? 1.f : a.proj[(size_t)row * a.ldp + a.g_off + (a.gate == LGATE_ELEM ? head * d + i : head)];
-        a.out[(size_t)row * a.ldo + head * d + i] = acc * gate / L;
+        a.out[(size_t)row * a.ldo + head * d + i] = acc * gate / L * a.out_scale;
     }
 }
 static size_t lay_attn_lds(int d, int e, bool own_v, int KT) {
@@ -1233,6 +1299,19 @@ constexpr int LL_ES = 32;
 // b_t = sum of the logarithms up to and including t (inside the chunk), all factors are exponentials of differences <= 0:
 //   o_t = S0^T (q_t * e^(b_t)) + sum_(s <= t) (sum_i q_t[i] k_s[i] e^(b_t[i] - b_s[i])) v_s,   S <- diag(e^(b_(n-1))) S0 + sum_s (k_s * e^(b_(n-1) - b_s)) v_s^T
 // LDS of the gated form: one more [C][d] array (the running logarithms)
+// operands of the linear-attention kernels at pass row `row`: the logarithm of the decay (per key channel, or one per head), the key
+// (times its per-token factor), the value column c of e (the last one the constant 1 when asked for)
+__device__ __forceinline__ float ll_ldec(const LLightArgs& a, int row, int head, int i) {
+    return a.head_decay ? a.ldec[(size_t)row * a.ldd + head] : a.ldec[(size_t)row * a.ldd + (size_t)head * a.d + i];
+}
+__device__ __forceinline__ float ll_key(const LLightArgs& a, int row, int head, int i) {
+    const float k = a.proj[(size_t)row * a.ldp + a.k_off + (size_t)head * a.d + i];
+    return a.kmul ? k * a.kmul[(size_t)row * a.ldd + head] : k;
+}
+__device__ __forceinline__ float ll_val(const LLightArgs& a, int row, int head, int c) {
+    if (a.ones_col) return c == a.e - 1 ? 1.f : a.proj[(size_t)row * a.ldp + a.v_off + (size_t)head * (a.e - 1) + c];
+    return a.proj[(size_t)row * a.ldp + a.v_off + (size_t)head * a.e + c];
+}
 template <bool GT>
 __device__ __forceinline__ void ll_cumsum(float* bs, int n, int d, int tid) {
     if (GT) {
@@ -1270,12 +1349,12 @@ __global__ __launch_bounds__(256) void lay_lightning_kernel(LLightArgs a, int C)
             const int t = idx / d, i = idx - t * d;
             const size_t base = (size_t)(sg.row0 + t0 + t) * a.ldp + (size_t)head * d + i;
             qs[idx] = a.proj[base + a.q_off] * a.qscale;
-            ks[idx] = a.proj[base + a.k_off];
-            if (GT) bs[idx] = a.ldec[(size_t)(sg.row0 + t0 + t) * a.ldd + (size_t)head * d + i];
+            ks[idx] = ll_key(a, sg.row0 + t0 + t, head, i);
+            if (GT) bs[idx] = ll_ldec(a, sg.row0 + t0 + t, head, i);
         }
         for (int idx = tid; idx < n * LL_ES; idx += 256) {
             const int t = idx / LL_ES, j = idx % LL_ES;
-            vs[idx] = j < ne ? a.proj[(size_t)(sg.row0 + t0 + t) * a.ldp + a.v_off + (size_t)head * e + j0 + j] : 0.f;
+            vs[idx] = j < ne ? ll_val(a, sg.row0 + t0 + t, head, j0 + j) : 0.f;
         }
         if (GT) { __syncthreads(); ll_cumsum<GT>(bs, n, d, tid); }
         __syncthreads();
@@ -1283,7 +1362,10 @@ __global__ __launch_bounds__(256) void lay_lightning_kernel(LLightArgs a, int C)
             const int t = idx / n, s = idx - t * n;
             float dot = 0.f;
             if (s <= t) {
-                if (GT) {
+                if (GT && a.head_decay) {
+                    for (int i = 0; i < d; ++i) dot = fmaf(qs[t * d + i], ks[s * d + i], dot);
+                    dot *= expf(bs[t * d] - bs[s * d]);
+                } else if (GT) {
                     for (int i = 0; i < d; ++i) dot = fmaf(qs[t * d + i] * ks[s * d + i], expf(bs[t * d + i] - bs[s * d + i]), dot);
                 } else {
                     for (int i = 0; i < d; ++i) dot = fmaf(qs[t * d + i], ks[s * d + i], dot);
@@ -1350,12 +1432,12 @@ __global__ __launch_bounds__(256) void lay_light_chunk_kv_kernel(LLightArgs a) {
     }
     for (int idx = tid; idx < n * d; idx += 256) {
         const int t = idx / d, i = idx - t * d;
-        ks[idx] = a.proj[(size_t)(sg.row0 + ch.y + t) * a.ldp + a.k_off + (size_t)head * d + i];
-        if (GT) bs[idx] = a.ldec[(size_t)(sg.row0 + ch.y + t) * a.ldd + (size_t)head * d + i];
+        ks[idx] = ll_key(a, sg.row0 + ch.y + t, head, i);
+        if (GT) bs[idx] = ll_ldec(a, sg.row0 + ch.y + t, head, i);
     }
     for (int idx = tid; idx < n * LL_ES; idx += 256) {
         const int t = idx / LL_ES, j = idx % LL_ES;
-        vs[idx] = j < ne ? a.proj[(size_t)(sg.row0 + ch.y + t) * a.ldp + a.v_off + (size_t)head * e + j0 + j] : 0.f;
+        vs[idx] = j < ne ? ll_val(a, sg.row0 + ch.y + t, head, j0 + j) : 0.f;
     }
     __syncthreads();
     if (GT) {
@@ -1429,7 +1511,7 @@ __global__ __launch_bounds__(256) void lay_light_chunk_out_kernel(LLightArgs a) 
         }
         for (int idx = tid; idx < n * LL_ES; idx += 256) {
             const int t = idx / LL_ES, j = idx % LL_ES;
-            vs[idx] = j < ne ? a.proj[(size_t)(sg.row0 + ch.y + t) * a.ldp + a.v_off + (size_t)head * e + j0 + j] : 0.f;
+            vs[idx] = j < ne ? ll_val(a, sg.row0 + ch.y + t, head, j0 + j) : 0.f;
         }
     };
     load_slice();
@@ -1437,8 +1519,8 @@ __global__ __launch_bounds__(256) void lay_light_chunk_out_kernel(LLightArgs a) 
         const int t = idx / d, i = idx - t * d;
         const size_t base = (size_t)(sg.row0 + ch.y + t) * a.ldp + (size_t)head * d + i;
         qs[idx] = a.proj[base + a.q_off] * a.qscale;
-        ks[t * ldk + i] = a.proj[base + a.k_off];
-        if (GT) bs[t * ldk + i] = a.ldec[(size_t)(sg.row0 + ch.y + t) * a.ldd + (size_t)head * d + i];
+        ks[t * ldk + i] = ll_key(a, sg.row0 + ch.y + t, head, i);
+        if (GT) bs[t * ldk + i] = ll_ldec(a, sg.row0 + ch.y + t, head, i);
     }
     __syncthreads();
     if (GT) {
@@ -1452,7 +1534,10 @@ __global__ __launch_bounds__(256) void lay_light_chunk_out_kernel(LLightArgs a) 
         const int t = idx / n, s = idx - t * n;
         float dot = 0.f;
         if (s <= t) {
-            if (GT) {
+            if (GT && a.head_decay) {      // one decay for all key channels: the plain dot product, one exponential
+                for (int i = 0; i < d; ++i) dot = fmaf(qs[t * d + i], ks[s * ldk + i], dot);
+                dot *= expf(bs[t * ldk] - bs[s * ldk]);
+            } else if (GT) {
                 for (int i = 0; i < d; ++i) dot = fmaf(qs[t * d + i] * ks[s * ldk + i], expf(bs[t * ldk + i] - bs[s * ldk + i]), dot);
             } else {
                 for (int i = 0; i < d; ++i) dot = fmaf(qs[t * d + i], ks[s * ldk + i], dot);
@@ -1499,12 +1584,12 @@ __global__ __launch_bounds__(256) void lay_light_decode_kernel(LLightArgs a) {
     const size_t prow = (size_t)sg.row0 * a.ldp;
     for (int i = tid; i < d; i += 256) {
         qk[i] = a.proj[prow + a.q_off + (size_t)head * d + i] * a.qscale;
-        qk[256 + i] = a.proj[prow + a.k_off + (size_t)head * d + i];
-        if (GT) qk[512 + i] = expf(a.ldec[(size_t)sg.row0 * a.ldd + (size_t)head * d + i]);
+        qk[256 + i] = ll_key(a, sg.row0, head, i);
+        if (GT) qk[512 + i] = expf(ll_ldec(a, sg.row0, head, i));
     }
     __syncthreads();
     const bool ok = j0 + j < e;
-    const float v = ok ? a.proj[prow + a.v_off + (size_t)head * e + j0 + j] : 0.f;
+    const float v = ok ? ll_val(a, sg.row0, head, j0 + j) : 0.f;
     float* st = a.state_pool + (size_t)sg.slot * a.slot_stride + a.st_off + (size_t)head * d * e + j0 + j;
     float o = 0.f;
     if (ok)
@@ -1556,11 +1641,86 @@ void launch_lay_lightning(const LLightArgs& a, hipStream_t s) {
 }
 
 // ------------------------------------------------------------------------------------------------------------------
+// matrix memory with exponential gates: S' = exp(lf + m - m') S + exp(li - m') k v^T, n' likewise with k alone, m' = max(lf + m, li),
+// o = S'^T q / (max(|n' . q|, exp(-m')) + 1e-6).  With the decay exp(lf + m - m') per head and token, the key factor exp(li - m') and a
+// constant 1 as one more value column (so that the state's last column is n) this is the gated linear attention above; what is
+// left are the gates with their running maximum (here) and the division, head norm and output gate (lay_memory_out).
+// ------------------------------------------------------------------------------------------------------------------
+// One wave per (sequence, head).  x -> max(x + lf, li) composes: after (a1, b1) then (a2, b2) it is x -> max(x + a1 + a2, max(b1 + a2, b2)),
+// so the running maximum of 64 tokens comes from a shuffle scan over the lanes; the portion's last m goes back to the state.
+__global__ __launch_bounds__(64) void lay_memory_gates_kernel(const float* __restrict__ proj, int ldp, int i_off, int f_off, float cap,
+                                                              float* __restrict__ ldec, float* __restrict__ kmul, float* __restrict__ mrun,
+                                                              float* __restrict__ state_pool, size_t slot_stride, size_t m_off,
+                                                              const LaySegDev* __restrict__ segs, int H) {
+    const LaySegDev sg = segs[blockIdx.x];
+    const int head = blockIdx.y, lane = threadIdx.x;
+    float* mp = state_pool + (size_t)sg.slot * slot_stride + m_off + head;
+    float m = *mp;
+    for (int t0 = 0; t0 < sg.n; t0 += 64) {
+        const int t = t0 + lane;
+        const bool ok = t < sg.n;
+        float li = -INFINITY, lf = 0.f;            // past the portion: the identity x -> x
+        if (ok) {
+            const float* pr = proj + (size_t)(sg.row0 + t) * ldp + head;
+            li = cap * tanhf(pr[i_off] / cap);
+            const float u = cap * tanhf(pr[f_off] / cap);
+            lf = fminf(u, 0.f) - log1pf(expf(-fabsf(u)));
+        }
+        float A = lf, B = li;
+        for (int off = 1; off < 64; off <<= 1) {
+            const float pa = __shfl_up(A, off), pb = __shfl_up(B, off);
+            if (lane >= off) { B = fmaxf(pb + A, B); A = pa + A; }
+        }
+        const float mt = fmaxf(m + A, B);
+        float mprev = __shfl_up(mt, 1);
+        if (lane == 0) mprev = m;
+        if (ok) {
+            const size_t o = (size_t)(sg.row0 + t) * H + head;
+            ldec[o] = lf + mprev - mt;
+            kmul[o] = expf(li - mt);
+            mrun[o] = mt;
+        }
+        m = __shfl(mt, min(63, sg.n - t0 - 1));
+    }
+    if (lane == 0) *mp = m;
+}
+void launch_lay_memory_gates(const float* proj, int ldp, int i_off, int f_off, float cap, float* ldec, float* kmul, float* mrun,
+                             float* state_pool, size_t slot_stride, size_t m_off, const LaySegDev* segs, int nseg, int H, hipStream_t s) {
+    if (nseg <= 0 || H <= 0) return;
+    hipLaunchKernelGGL(lay_memory_gates_kernel, dim3((unsigned)nseg, (unsigned)H), dim3(64), 0, s, proj, ldp, i_off, f_off, cap, ldec, kmul, mrun,
+                       state_pool, slot_stride, m_off, segs, H);
+}
+// one wave per (row, head)
+__global__ __launch_bounds__(256) void lay_memory_out_kernel(const float* __restrict__ o, const float* __restrict__ mrun,
+                                                             const float* __restrict__ gate, int ldg, const float* __restrict__ w,
+                                                             float* __restrict__ out, int ldo, int H, int e, float eps, float out_scale) {
+    const int r = blockIdx.x, lane = threadIdx.x & 63;
+    const int head = (int)blockIdx.y * 4 + (int)(threadIdx.x >> 6);
+    if (head >= H) return;
+    const float* oh = o + ((size_t)r * H + head) * (e + 1);
+    const float den = fmaxf(fabsf(oh[e]), expf(-mrun[(size_t)r * H + head])) + 1e-6f;
+    float ss = 0.f;
+    for (int c = lane; c < e; c += 64) { const float v = oh[c] / den; ss += v * v; }
+    ss = wave_sum(ss);
+    const float rs = 1.f / sqrtf(ss / (float)e + eps);
+    for (int c = lane; c < e; c += 64)
+        out[(size_t)r * ldo + head * e + c] = oh[c] / den * rs * w[head * e + c] * gate[(size_t)r * ldg + head * e + c] * out_scale;
+}
+void launch_lay_memory_out(const float* o, const float* mrun, const float* gate, int ldg, const float* w, float* out, int ldo, int T, int H,
+                           int e, float eps, float out_scale, hipStream_t s) {
+    if (T <= 0 || H <= 0) return;
+    hipLaunchKernelGGL(lay_memory_out_kernel, dim3((unsigned)T, (unsigned)((H + 3) / 4)), dim3(256), 0, s, o, mrun, gate, ldg, w, out, ldo, H, e,
+                       eps, out_scale);
+}
+
+// ------------------------------------------------------------------------------------------------------------------
 // mixture of experts: router + counting sort
 // ------------------------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void lay_router_kernel(const float* __restrict__ h, const uint16_t* __restrict__ wr, int32_t* __restrict__ sel,
-                                                         float* __restrict__ wsel, int W, int E, int top) {
-    extern __shared__ float zs[];          // [E]
+                                                         float* __restrict__ wsel, int W, int E, int top, RouterSpec rs,
+                                                         const float* __restrict__ correction, int slots) {
+    extern __shared__ float zs[];          // [E] logits, then choice scores; [E] scores
+    float* sc = zs + E;
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float* hr = h + (size_t)t * W;
     for (int ex = wave; ex < E; ex += 4) {
@@ -1571,6 +1731,31 @@ __global__ __launch_bounds__(256) void lay_router_kernel(const float* __restrict
     }
     __syncthreads();
     if (threadIdx.x == 0) {
+        // scores; the choice goes by score + correction (plain sigmoid scores: by the logits themselves, the same order)
+        if (rs.softmax) {
+            float mx = -INFINITY, sum = 0.f;
+            for (int ex = 0; ex < E; ++ex) mx = fmaxf(mx, zs[ex]);
+            for (int ex = 0; ex < E; ++ex) { sc[ex] = expf(zs[ex] - mx); sum += sc[ex]; }
+            for (int ex = 0; ex < E; ++ex) sc[ex] /= sum;
+        } else
+            for (int ex = 0; ex < E; ++ex) sc[ex] = 1.f / (1.f + expf(-zs[ex]));
+        if (rs.softmax || correction)
+            for (int ex = 0; ex < E; ++ex) zs[ex] = sc[ex] + (correction ? correction[ex] : 0.f);
+        if (rs.groups > 1) {               // keep the best groups: every pass removes the worst remaining one
+            const int per = E / rs.groups;
+            for (int drop = 0; drop < rs.groups - rs.keep_groups; ++drop) {
+                int worst = -1; float wv = 0.f;
+                for (int g = rs.groups - 1; g >= 0; --g) {     // among equals the later group goes first
+                    float best = -INFINITY; bool live = false;
+                    for (int j = 0; j < per; ++j) { const float c = zs[g * per + j]; if (c != -INFINITY) live = true; best = fmaxf(best, c); }
+                    if (!live) continue;
+                    if (worst < 0 || best < wv) { worst = g; wv = best; }
+                }
+                if (worst < 0) break;
+                for (int j = 0; j < per; ++j) zs[worst * per + j] = -INFINITY;
+            }
+        }
+        float wsum = 0.f;
         for (int k = 0; k < top; ++k) {
             int best = -1; float bz = 0.f;
             for (int ex = 0; ex < E; ++ex) {
@@ -1578,20 +1763,26 @@ __global__ __launch_bounds__(256) void lay_router_kernel(const float* __restrict
                 if (z == -INFINITY) continue;
                 if (best < 0 || z > bz) { best = ex; bz = z; }
             }
-            if (best < 0) { best = 0; bz = 0.f; }
+            if (best < 0) { best = 0; }
             sel[(size_t)t * top + k] = best;
-            wsel[(size_t)t * top + k] = 1.f / (1.f + expf(-bz));
+            wsel[(size_t)t * slots + k] = sc[best];
+            wsum += sc[best];
             zs[best] = -INFINITY;
         }
+        if (rs.normalise) for (int k = 0; k < top; ++k) wsel[(size_t)t * slots + k] /= wsum + 1e-20f;
+        for (int k = top; k < slots; ++k) wsel[(size_t)t * slots + k] = 1.f;
     }
 }
-void launch_lay_router(const float* h, const uint16_t* wr, int32_t* sel, float* wsel, int T, int W, int E, int top, hipStream_t s) {
+void launch_lay_router(const float* h, const uint16_t* wr, int32_t* sel, float* wsel, int T, int W, int E, int top, hipStream_t s,
+                       const RouterSpec* rs, const float* correction, int slots) {
     if (T <= 0) return;
-    hipLaunchKernelGGL(lay_router_kernel, dim3((unsigned)T), dim3(256), (size_t)E * sizeof(float), s, h, wr, sel, wsel, W, E, top);
+    const RouterSpec r = rs ? *rs : RouterSpec();
+    hipLaunchKernelGGL(lay_router_kernel, dim3((unsigned)T), dim3(256), (size_t)2 * E * sizeof(float), s, h, wr, sel, wsel, W, E, top, r,
+                       r.correction ? correction : nullptr, slots > top ? slots : top);
 }
 
 __global__ __launch_bounds__(1024) void lay_moe_plan_kernel(const int32_t* __restrict__ sel, int32_t* __restrict__ off, int32_t* __restrict__ srt,
-                                                            int n, int E) {
+                                                            int n, int E, int top, int slots) {
     extern __shared__ int cnt[];           // [E] counts, then cursors
     for (int i = threadIdx.x; i < E; i += 1024) cnt[i] = 0;
     __syncthreads();
@@ -1603,10 +1794,21 @@ __global__ __launch_bounds__(1024) void lay_moe_plan_kernel(const int32_t* __res
         off[E] = run;
     }
     __syncthreads();
-    for (int p = threadIdx.x; p < n; p += 1024) srt[atomicAdd(&cnt[sel[p]], 1)] = p;
+    for (int p = threadIdx.x; p < n; p += 1024) srt[atomicAdd(&cnt[sel[p]], 1)] = (p / top) * slots + p % top;
 }
-void launch_lay_moe_plan(const int32_t* sel, int32_t* off, int32_t* srt, int n, int E, hipStream_t s) {
-    hipLaunchKernelGGL(lay_moe_plan_kernel, dim3(1), dim3(1024), (size_t)E * sizeof(int), s, sel, off, srt, n, E);
+void launch_lay_moe_plan(const int32_t* sel, int32_t* off, int32_t* srt, int n, int E, hipStream_t s, int top, int slots) {
+    hipLaunchKernelGGL(lay_moe_plan_kernel, dim3(1), dim3(1024), (size_t)E * sizeof(int), s, sel, off, srt, n, E, top, slots);
+}
+__global__ __launch_bounds__(256) void lay_moe_identity_kernel(const int32_t* __restrict__ sel, const float* __restrict__ h, float* __restrict__ ys,
+                                                               int W, int top, int slots, int n_real) {
+    const int p = blockIdx.x;
+    if (sel[p] < n_real) return;
+    const int t = p / top, k = p - t * top;
+    for (int c = threadIdx.x; c < W; c += 256) ys[((size_t)t * slots + k) * W + c] = h[(size_t)t * W + c];
+}
+void launch_lay_moe_identity(const int32_t* sel, const float* h, float* ys, int T, int W, int top, int slots, int n_real, hipStream_t s) {
+    if (T <= 0 || top <= 0) return;
+    hipLaunchKernelGGL(lay_moe_identity_kernel, dim3((unsigned)(T * top)), dim3(256), 0, s, sel, h, ys, W, top, slots, n_real);
 }
 
 // arg-max of every row, lowest index among equals

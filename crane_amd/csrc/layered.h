@@ -7,7 +7,13 @@
 //     front of the mixer (the two-tap case of the short convolution), softmax attention inside position chunks with a linear
 //     distance bias / a sink term in the denominator / an element-wise sigmoid gate / keys and values borrowed from an earlier
 //     layer, latent attention (low-rank queries, one cached latent + one rotated key part per token, YaRN-scaled rotation), gated
-//     linear attention with a data-dependent decay per key channel, dense squared-ReLU feed-forwards.
+//     linear attention with a data-dependent decay per key channel, dense squared-ReLU feed-forwards;
+//   Gibipel -- no norm in front of a sublayer, a one-number RMS norm on its output (x += g * unit(sublayer(x))); two mixers side by
+//     side on the same input, their outputs scaled and summed: softmax attention over a sliding window plus one mean key / mean
+//     value per block of positions that lies wholly in front of the window (query / key RMS norm over all heads at once,
+//     half-split rotation with banded frequency stretching, sink), and a matrix memory with exponential input / forget gates
+//     (running-maximum stabiliser, normaliser vector); mixture-of-experts feed-forwards with a softmax router (choice by score +
+//     correction inside the best groups of neighbours, identity experts, a shared expert).
 // The mechanisms are kernels with their constants as arguments (kernels_layered.hip); the per-layer plumbing and the step function
 // over mixed batches (prompt portions beside single decode tokens) are in model_layered.cpp.
 #pragma once
@@ -19,7 +25,8 @@
 
 namespace cm {
 
-enum { LMIX_ATTN = 0, LMIX_LIGHTNING = 1, LMIX_LATENT = 2, LMIX_GLA = 3 };
+// LMIX_SIDE: the mixers in LayerSpec::side run side by side on the layer's input; LMIX_MEMORY: matrix memory with exponential gates
+enum { LMIX_ATTN = 0, LMIX_LIGHTNING = 1, LMIX_LATENT = 2, LMIX_GLA = 3, LMIX_MEMORY = 4, LMIX_SIDE = 5 };
 enum { LMLP_NONE = 0, LMLP_DENSE = 1, LMLP_MOE = 2 };
 // LACT_RELU2: max(v, 0)^2;  LACT_LOGSIG: act_param * ln(sigmoid(v)) (the logarithm of a decay sigmoid(v)^act_param)
 enum { LACT_NONE = 0, LACT_SILU = 1, LACT_SIGMOID = 2, LACT_GELU_TANH = 3, LACT_RELU2 = 4, LACT_LOGSIG = 5 };
@@ -28,12 +35,26 @@ enum { LBIAS_NONE = 0, LBIAS_LOG = 1, LBIAS_LINEAR = 2 };
 // gate on the attention output: none | one value per head at g_off + head | one per element at g_off + head e + i
 enum { LGATE_NONE = 0, LGATE_HEAD = 1, LGATE_ELEM = 2 };
 
-// rotation of consecutive pairs (2i, 2i + 1) of the first `dims` elements of a vector by the angle position * freq[i]
+// rotation of pairs of the first `dims` elements of a vector by the angle position * freq[i]: consecutive pairs (2i, 2i + 1), or
+// (half) element i with element i + dims / 2
 struct RotSpec {
     int dims = 0;
     double base = 10000.0;
     bool yarn = false;
     double factor = 1.0, original = 0.0, fast = 32.0, slow = 1.0;
+    bool half = false;
+    // banded stretching: wavelengths above original / low are stretched by factor, those below original / high are kept, the band
+    // between blends the two frequencies linearly in original / wavelength
+    bool banded = false;
+    double low = 1.0, high = 4.0;
+};
+// how a router turns its logits into choices and weights
+struct RouterSpec {
+    bool softmax = false;              // scores: softmax over all outputs (false: sigmoid of each)
+    bool correction = false;           // a learned vector joins the scores for the choice only
+    int groups = 1, keep_groups = 1;   // outputs form `groups` equal groups of neighbours; only the keep_groups best (by their largest choice score) can be chosen
+    bool normalise = false;            // weights divided by their sum
+    int identity = 0;                  // the last `identity` outputs pass the input through (no matrices)
 };
 
 // one entry of config "layers"
@@ -54,6 +75,13 @@ struct LayerSpec {
     int mlp = LMLP_NONE, ff = 0, experts = 0, top = 0;
     bool gated_ff = true;              // dense: act(gate) * up (false: act(up) alone)
     int ff_act = LACT_GELU_TANH;
+    long long pool = 0;                // attention: blocks of `pool` positions wholly in front of the window are seen through their mean key / value
+    bool qk_norm = false, qkv_bias = false;   // attention: RMS norm of all query (key) heads at once; biases on q, k, v
+    float gate_cap = 0.f;              // matrix memory: gate pre-activations pass cap * tanh(z / cap)
+    RouterSpec router;
+    int shared_ff = 0;                 // mixture of experts: inner size of the expert every token uses (0: none)
+    std::vector<LayerSpec> side;       // LMIX_SIDE: the mixers, each scaled by its side_scale
+    float side_scale = 1.f;
 };
 
 // device-side weights of one layer (bf16 matrices [out, in], f32 vectors)
@@ -85,6 +113,14 @@ struct LayeredLayerW {
     size_t k_pool_off = 0, k_page_bytes = 0;         // this layer's key pages inside the pool
     size_t st_off = 0;                               // lightning state offset inside a slot of the state pool (floats)
     size_t c1_off = 0, c2_off = 0;                   // convolution tails inside a slot of the conv pool (floats)
+    float *q_norm = nullptr, *k_norm = nullptr;      // attention: [H d], [G d] weights of the norm over all heads
+    size_t pk_pool_off = 0, pv_pool_off = 0, pk_page_bytes = 0, pv_page_bytes = 0;   // mean key / value rows of the position blocks
+    int pool_rows = 0;                               // ... rows per page: the blocks whose last position lies in the page
+    int i_off = 0, f_off = 0;                        // matrix memory: gate pre-activations inside the projection row
+    float* correction = nullptr;                     // router: [outputs]
+    uint16_t *sh_gate = nullptr, *sh_up = nullptr, *sh_down = nullptr;   // shared expert
+    int o_col = 0;                                   // side mixers: first column of this mixer's heads in the joint output projection's input
+    std::vector<LayeredLayerW> side;
 };
 
 // rows [row0, row0 + n) of a pass are positions start_pos.. of the sequence in `slot`; its page table starts at bt_off
@@ -114,7 +150,7 @@ void launch_lgemm(const LGemmArgs& a, bool bf16, int groups, hipStream_t s);
 void launch_lay_act_cols(float* C, int ldc, int M, int N, int act, int act2, int split, hipStream_t s, float param = 1.f);
 void launch_lay_act_mul(const float* g, const float* u, float* out, size_t n, int act, hipStream_t s);
 void launch_lay_round_rows(const float* x, int ldx, uint16_t* out, int M, int K, hipStream_t s);
-void launch_lay_embed_rows(const uint16_t* emb, const uint32_t* ids, float* x, int T, int W, int V, hipStream_t s);
+void launch_lay_embed_rows(const uint16_t* emb, const uint32_t* ids, float* x, int T, int W, int V, hipStream_t s, float scale = 1.f);
 void launch_lay_rms_rows(const float* x, const int32_t* rows, const float* w, float* out, int n_rows, int W, float eps, hipStream_t s);
 // two norms of the same rows (one root mean square, two weights)
 void launch_lay_rms_rows2(const float* x, const float* w1, const float* w2, float* out1, float* out2, int T, int W, float eps, hipStream_t s);
@@ -128,9 +164,9 @@ void launch_lay_add_norm2_shift_decode(float* x, const float* y1, const float* y
 // x += y1 + y2 (y2 may be null)
 void launch_lay_add_rows(float* x, const float* y1, const float* y2, size_t n, hipStream_t s);
 // pairs (2i, 2i + 1), i < dims / 2, of `nvec` vectors per row (vector v at src + r lds + v vstride) turned by position * freq[i];
-// cos and sin times mag; elements past dims are copied.  dst may be src.
+// cos and sin times mag; elements past dims are copied.  dst may be src.  half: the pairs are (i, i + dims / 2) instead.
 void launch_lay_rope(const float* src, int lds, int s_vstride, float* dst, int ldd, int d_vstride, int nvec, int len, int dims,
-                     const float* freq, float mag, const LaySegDev* segs, const int32_t* rowseg, int T, hipStream_t s);
+                     const float* freq, float mag, const LaySegDev* segs, const int32_t* rowseg, int T, hipStream_t s, bool half = false);
 // out = h + conv(h) over time per channel; the taps - 1 inputs before a portion come from the sequence's tail in conv_pool
 void launch_lay_canon(const float* h, float* out, const float* cw, const float* conv_pool, size_t slot_stride, size_t off,
                       const LaySegDev* segs, const int32_t* rowseg, int T, int W, int taps, hipStream_t s);
@@ -162,9 +198,18 @@ struct LAttnArgs {
     // few query tiles, many keys (decode steps): nsplit blocks per tile share its key tiles and a merge launch follows;
     // part_o [ntiles][G][nsplit][16][d], part_ml [ntiles][G][nsplit][16][2].  nsplit <= 1 or null scratch: one block per tile
     int nsplit = 1; float* part_o = nullptr; float* part_ml = nullptr;
+    // pool > 0: block b of `pool` positions is seen by position i through one mean key and one mean value when its last position
+    // b pool + pool - 1 <= i - win; rows [n_pages][G][pool_rows][d] / [e] (lay_pool_append), in front of the window in the key walk
+    long long pool = 0; const void* pk_pool = nullptr; const void* pv_pool = nullptr; int pool_rows = 0;
+    float out_scale = 1.f;                           // factor on the output
 };
 void launch_lay_k_append(const float* proj, int ldp, int k_off, void* kpool, int kvt, const int32_t* bt, const LaySegDev* segs,
                          const int32_t* rowseg, int T, int G, int d, int page, hipStream_t s);
+// mean key (and value) rows of the position blocks that the pass completes: block b of `pool` positions lives in the page of its
+// last position, row b - (first block that ends in that page).  Reads the cached rows, so it follows lay_k_append.
+void launch_lay_pool_append(const void* kpool, void* pk_pool, int kvt, const int32_t* bt, const LaySegDev* segs, const int32_t* rowseg, int T,
+                            int G, int d, int page, int pool, int pool_rows, hipStream_t s);
+inline int lay_pool_rows(int page, long long pool) { return pool >= page ? 1 : (int)((page + pool - 1) / pool); }
 void launch_lay_attn(const LAttnArgs& a, int kvt, hipStream_t s);    // kvt: KV_BF16 | KV_F32
 bool lay_attn_fits(int d, int e, bool own_v);                         // sizes the kernel can hold in LDS and registers
 int lay_attn_key_tile(int d, int e, bool own_v);                      // keys per tile of lay_attn_kernel at these sizes (64 or 32)
@@ -189,6 +234,10 @@ struct LLightArgs {
     const float* ldec = nullptr; int ldd = 0;
     float qscale = 1.f;          // q is multiplied by this
     float* D = nullptr;          // gated chunk-parallel form: [nchunks][H][d] decay of a whole chunk
+    // one decay per head and token instead of one per key channel: ldec[t ldd + head] (head_decay), and a factor on the key:
+    // k_t * kmul[t ldd + head].  ones_col: the last of the e value columns is the constant 1 (the projection row holds e - 1 per
+    // head), so that the state's last column carries sum_s decay(s..t) k_s -- the normaliser of a matrix memory
+    bool head_decay = false; const float* kmul = nullptr; bool ones_col = false;
 };
 constexpr int LAY_LIGHT_CHUNK = 32;
 void launch_lay_lightning(const LLightArgs& a, hipStream_t s);
@@ -197,10 +246,24 @@ void launch_lay_lightning(const LLightArgs& a, hipStream_t s);
 void launch_lay_rms_gate(const float* o, const float* gate, int ldg, const float* w, float* out, int T, int N, float eps, hipStream_t s,
                          int group = 0, bool shared_w = false);
 
-// router: z = h . Wr^T in f32, the `top` largest (lowest index first among equals) -> sel [T top], wsel = sigmoid(z)
-void launch_lay_router(const float* h, const uint16_t* wr, int32_t* sel, float* wsel, int T, int W, int E, int top, hipStream_t s);
-// counting sort of the T top (token, choice) pairs by expert: off [E + 1], srt [T top]
-void launch_lay_moe_plan(const int32_t* sel, int32_t* off, int32_t* srt, int n, int E, hipStream_t s);
+// router: z = h . Wr^T in f32 over E outputs, scores by rs (sigmoid of each / softmax over all), the `top` largest choice scores
+// (score + correction, inside the best groups; lowest index first among equals) -> sel [T top], wsel [T slots] = their scores
+// (normalised when asked); slots > top: the remaining weights are 1 (rows that every token uses, e.g. a shared expert)
+void launch_lay_router(const float* h, const uint16_t* wr, int32_t* sel, float* wsel, int T, int W, int E, int top, hipStream_t s,
+                       const RouterSpec* rs = nullptr, const float* correction = nullptr, int slots = 0);
+// counting sort of the T top (token, choice) pairs by expert: off [E + 1], srt [T top] = token * slots + choice
+void launch_lay_moe_plan(const int32_t* sel, int32_t* off, int32_t* srt, int n, int E, hipStream_t s, int top = 1, int slots = 1);
+// rows of the identity experts: ys[token * slots + choice] = h[token] where sel >= n_real
+void launch_lay_moe_identity(const int32_t* sel, const float* h, float* ys, int T, int W, int top, int slots, int n_real, hipStream_t s);
+
+// matrix memory, gates: per (sequence, head) over the portion's tokens, from the pre-activations zi, zf at proj[t ldp + i_off / f_off + head]
+//   li = cap tanh(zi / cap), lf = ln sigmoid(cap tanh(zf / cap)), m' = max(lf + m, li)  (m: per-sequence state at mstate, [H])
+//   ldec[t H + head] = lf + m - m' (<= 0), kmul[t H + head] = exp(li - m') (<= 1), mrun[t H + head] = m'
+void launch_lay_memory_gates(const float* proj, int ldp, int i_off, int f_off, float cap, float* ldec, float* kmul, float* mrun,
+                             float* state_pool, size_t slot_stride, size_t m_off, const LaySegDev* segs, int nseg, int H, hipStream_t s);
+// matrix memory, output: o [T][H (e + 1)] = [S^T q | n . q] -> out[t ldo + head e + c] = unit_rms_e(o_c / (max(|n . q|, exp(-m')) + 1e-6)) * w[head e + c] * gate * out_scale
+void launch_lay_memory_out(const float* o, const float* mrun, const float* gate, int ldg, const float* w, float* out, int ldo, int T, int H,
+                           int e, float eps, float out_scale, hipStream_t s);
 constexpr int LAY_ARGMAX_PARTS = 64;
 // pv / pi: [n_rows][LAY_ARGMAX_PARTS] scratch of the two-launch form for wide rows (null: one block per row)
 void launch_lay_argmax_rows(const float* logits, int ld, int V, uint32_t* out, int n_rows, float* pv, int* pi, hipStream_t s);

@@ -25,6 +25,11 @@ struct Layered {
     // Mononex: x += mixer(shift(norm1 x)) + ff(norm2 x), no norm behind the sublayers; Korupel: one sublayer after the other,
     // a norm on each side
     bool parallel = false;
+    // Gibipel: a sublayer reads the residual itself and a one-number norm sits on its output; embedding and logits are scaled
+    bool post_only = false;
+    float embed_scale = 1.f, logit_scale = 1.f;
+    int max_mh = 0, max_sff = 0, max_slots = 1;   // matrix-memory heads, shared expert size, rows per token of an expert combine
+    float *KM = nullptr, *MR = nullptr, *HS = nullptr;   // matrix memory: key factor and running maximum per token and head; shared expert's inner rows
     int max_q = 0, max_qa = 0, max_cq = 0, max_ld = 0, max_e = 0;
     bool f32 = false;                  // number format of the projections and the key cache
     float* final_norm = nullptr;
@@ -116,7 +121,22 @@ static void parse_mlp(const cmjson::Value* ml, LayerSpec& sp, bool moe_ok) {
         sp.ff = (int)ex->integer("ff", 0);
         sp.experts = (int)rt->integer("experts", 0);
         sp.top = (int)rt->integer("top", 0);
-        if (sp.experts <= 0 || sp.top <= 0 || sp.top > sp.experts || sp.experts > 4096) throw CmError(CM_ERR_INVALID, "router.experts / router.top");
+        sp.router.identity = (int)rt->integer("identity", 0);
+        if (const cmjson::Value* gr = rt->get("groups"))
+            if (gr->kind == cmjson::Value::Obj) {
+                sp.router.groups = (int)gr->integer("count", 1);
+                sp.router.keep_groups = (int)gr->integer("keep", sp.router.groups);
+            }
+        const int outs = sp.experts + sp.router.identity;
+        if (sp.experts <= 0 || sp.top <= 0 || sp.router.identity < 0 || sp.top > outs || outs > 4096) throw CmError(CM_ERR_INVALID, "router.experts / router.top");
+        if (sp.router.groups <= 0 || outs % sp.router.groups || sp.router.keep_groups <= 0 || sp.router.keep_groups > sp.router.groups ||
+            sp.top > outs / sp.router.groups * sp.router.keep_groups)
+            throw CmError(CM_ERR_INVALID, "router.groups");
+        if (const cmjson::Value* sh = ml->get("shared"))
+            if (sh->kind == cmjson::Value::Obj) {
+                sp.shared_ff = (int)sh->integer("ff", 0);
+                if (sp.shared_ff <= 0) throw CmError(CM_ERR_IO, "config.json: shared.ff");
+            }
     } else throw CmError(CM_ERR_UNSUPPORTED, "mlp.kind '" + kind + "' not implemented");
     if (sp.ff <= 0) throw CmError(CM_ERR_IO, "config.json: ff");
 }
@@ -224,19 +244,89 @@ static void parse_mononex_layer(const cmjson::Value& e, LayerSpec& sp, const std
     sp.gated_ff = false; sp.ff_act = LACT_RELU2;
 }
 
+// Gibipel: layer type "parallel" = "mixer": {"left": window attention with pooled blocks, "right": matrix memory, "left_scale",
+// "right_scale"}; "mlp": mixture of experts with a softmax router ("identity", "groups": {"count", "keep"}, tensor "correction") and
+// an optional "shared" expert
+static void parse_gibipel_layer(const cmjson::Value& e, LayerSpec& sp) {
+    const std::string type = e.string("type", "");
+    if (type != "parallel") throw CmError(CM_ERR_UNSUPPORTED, "layer type '" + type + "' not implemented");
+    const cmjson::Value* mx = e.get("mixer");
+    const cmjson::Value* lf = mx ? mx->get("left") : nullptr;
+    const cmjson::Value* rg = mx ? mx->get("right") : nullptr;
+    need(lf && rg && lf->kind == cmjson::Value::Obj && rg->kind == cmjson::Value::Obj, "parallel layer without mixer.left / mixer.right");
+    sp.mixer = LMIX_SIDE;
+    sp.side.resize(2);
+    {
+        LayerSpec& a = sp.side[0];
+        a.mixer = LMIX_ATTN;
+        a.side_scale = (float)mx->number("left_scale", 1.0);
+        a.heads = (int)lf->integer("heads", 0);
+        a.kv_heads = (int)lf->integer("kv_heads", a.heads);
+        a.dim = (int)lf->integer("dim", 0);
+        a.vdim = (int)lf->integer("vdim", a.dim);
+        need(a.heads > 0 && a.dim > 0 && a.vdim > 0 && a.kv_heads > 0 && a.heads % a.kv_heads == 0, "left mixer sizes");
+        a.scale = (float)lf->number("scale", 1.0 / std::sqrt((double)a.dim));
+        a.win = 1ll << 40; a.keep = 0;
+        if (const cmjson::Value* mk = lf->get("mask"))
+            if (mk->kind == cmjson::Value::Obj) {
+                a.win = mk->integer("size", a.win);
+                a.pool = mk->integer("pool", 0);
+                need(a.win > 0 && a.pool >= 0, "mask.size / mask.pool");
+            }
+        if (const cmjson::Value* rt = lf->get("rot"))
+            if (rt->kind == cmjson::Value::Obj) {
+                a.rot.half = true;
+                a.rot.dims = (int)rt->integer("dims", a.dim);
+                a.rot.base = rt->number("base", 10000.0);
+                if (const cmjson::Value* sc = rt->get("scaling"))
+                    if (sc->kind == cmjson::Value::Obj) {
+                        a.rot.banded = true;
+                        a.rot.factor = sc->number("factor", 1.0);
+                        a.rot.low = sc->number("low", 1.0);
+                        a.rot.high = sc->number("high", 4.0);
+                        a.rot.original = sc->number("original", 0.0);
+                        need(a.rot.factor > 0 && a.rot.original > 0 && a.rot.low > 0 && a.rot.high > a.rot.low, "rot.scaling");
+                    }
+                need(a.rot.dims >= 0 && a.rot.dims <= a.dim && a.rot.dims % 2 == 0 && a.rot.base > 1.0, "rot.dims / rot.base");
+            }
+        a.bias = LBIAS_NONE; a.gate = LGATE_NONE; a.sink = true; a.own_v = true; a.qk_norm = true; a.qkv_bias = true;
+        need(lay_attn_fits(a.dim, a.vdim, true), "attention head sizes too large");
+    }
+    {
+        LayerSpec& b = sp.side[1];
+        b.mixer = LMIX_MEMORY;
+        b.side_scale = (float)mx->number("right_scale", 1.0);
+        b.heads = (int)rg->integer("heads", 0);
+        b.kv_heads = b.heads;
+        b.dim = (int)rg->integer("dim", 0);
+        b.vdim = (int)rg->integer("vdim", b.dim);
+        b.gate_cap = (float)rg->number("gate_cap", 15.0);
+        need(b.heads > 0 && b.dim > 0 && b.vdim > 0 && b.gate_cap > 0.f, "right mixer sizes");
+        if (b.dim > 256) throw CmError(CM_ERR_UNSUPPORTED, "matrix memory head size above 256");
+    }
+    parse_mlp(e.get("mlp"), sp, true);
+    sp.router.softmax = true; sp.router.correction = true; sp.router.normalise = true;
+}
+
 // config.json of a layer-list decoder: "architecture", "vocab", "width", "norm".eps and "layers": [{"type", "mixer": {...}, "mlp"}]
 void Model::init_layered_config(const cmjson::Value& root) {
     const std::string arch = root.string("architecture", "");
-    if (arch != "Korupel" && arch != "Mononex") throw CmError(CM_ERR_UNSUPPORTED, "architecture '" + arch + "' not implemented (Korupel, Mononex)");
+    if (arch != "Korupel" && arch != "Mononex" && arch != "Gibipel")
+        throw CmError(CM_ERR_UNSUPPORTED, "architecture '" + arch + "' not implemented (Korupel, Mononex, Gibipel)");
     layered = true;
     lay.reset(new Layered());
     Layered& L = *lay;
     L.parallel = arch == "Mononex";
-    cfg.model_type = L.parallel ? "mononex" : "korupel";
+    L.post_only = arch == "Gibipel";
+    cfg.model_type = L.parallel ? "mononex" : (L.post_only ? "gibipel" : "korupel");
+    if (L.post_only) {
+        if (const cmjson::Value* em = root.get("embedding")) L.embed_scale = (float)em->number("scale", 1.0);
+        L.logit_scale = (float)root.number("logit_scale", 1.0);
+    }
     cfg.V = (int)root.integer("vocab", 0);
     cfg.H = (int)root.integer("width", 0);
     if (const cmjson::Value* n = root.get("norm")) cfg.eps = (float)n->number("eps", 1e-6);
-    if (!L.parallel) {
+    if (!L.parallel && !L.post_only) {
         if (const cmjson::Value* c = root.get("canon")) L.taps = (int)c->integer("taps", 0);
         L.mult = (float)root.number("residual_mult", 1.0);
     }
@@ -247,6 +337,7 @@ void Model::init_layered_config(const cmjson::Value& root) {
     for (auto& e : ls->arr) {
         LayerSpec sp;
         if (L.parallel) parse_mononex_layer(*e, sp, L.spec);
+        else if (L.post_only) parse_gibipel_layer(*e, sp);
         else parse_korupel_layer(*e, sp);
         L.spec.push_back(sp);
     }
@@ -353,6 +444,14 @@ static std::vector<float> rot_frequencies(const RotSpec& r, float* mag) {
     }
     for (int i = 0; i < half; ++i) {
         double fi = std::pow(r.base, -2.0 * i / r.dims);
+        if (r.banded) {
+            const double wavelength = 6.283185307179586476925286766559 / fi;
+            if (wavelength > r.original / r.low) fi /= r.factor;
+            else if (wavelength >= r.original / r.high) {
+                const double t = (r.original / wavelength - r.low) / (r.high - r.low);
+                fi = (1.0 - t) * fi / r.factor + t * fi;
+            }
+        }
         if (r.yarn) {
             const double ramp = std::min(1.0, std::max(0.0, (i - lo) / std::max(hi - lo, 0.001)));
             fi = fi / r.factor * ramp + fi * (1.0 - ramp);
@@ -363,10 +462,12 @@ static std::vector<float> rot_frequencies(const RotSpec& r, float* mag) {
 }
 
 static void build_mononex(Model& m, LaySource& src);
+static void build_gibipel(Model& m, LaySource& src);
 
 static void build_layered(Model& m, LaySource& src) {
     Layered& L = *m.lay;
     if (L.parallel) { build_mononex(m, src); return; }
+    if (L.post_only) { build_gibipel(m, src); return; }
     const size_t W = (size_t)m.cfg.H, V = (size_t)m.cfg.V;
     const float ws = 1.0f / std::sqrt((float)W);
     m.embed = up_bf16(m, src.get("embed", V * W, 1.0f, 0.f));
@@ -523,6 +624,112 @@ static void build_mononex(Model& m, LaySource& src) {
     m.lm_head = L.head;
 }
 
+// experts' matrices back to back, router, correction, shared expert (the Gibipel feed-forward)
+static void build_experts(Model& m, LaySource& src, const std::string& p, const LayerSpec& sp, LayeredLayerW& w) {
+    const size_t W = (size_t)m.cfg.H, ff = (size_t)sp.ff;
+    const float ws = 1.0f / std::sqrt((float)W), fs = 1.0f / std::sqrt((float)ff);
+    std::vector<float> g, u, dn;
+    for (int ex = 0; ex < sp.experts; ++ex) {
+        const std::string q = p + "mlp.e" + std::to_string(ex) + ".";
+        append(g, src.get(q + "gate", ff * W, ws, 0.f));
+        append(u, src.get(q + "up", ff * W, ws, 0.f));
+        append(dn, src.get(q + "down", W * ff, fs, 0.f));
+    }
+    w.gate = up_bf16(m, g); w.up = up_bf16(m, u); w.down = up_bf16(m, dn);
+    const size_t outs = (size_t)(sp.experts + sp.router.identity);
+    w.router = up_bf16(m, src.get(p + "mlp.router", outs * W, ws, 0.f));
+    if (sp.router.correction) w.correction = up_f32(m, src.get(p + "mlp.correction", outs, 0.02f, 0.f));
+    if (sp.shared_ff > 0) {
+        const size_t sf = (size_t)sp.shared_ff;
+        w.sh_gate = up_bf16(m, src.get(p + "mlp.shared.gate", sf * W, ws, 0.f));
+        w.sh_up = up_bf16(m, src.get(p + "mlp.shared.up", sf * W, ws, 0.f));
+        w.sh_down = up_bf16(m, src.get(p + "mlp.shared.down", W * sf, 1.0f / std::sqrt((float)sf), 0.f));
+    }
+}
+
+static void build_gibipel(Model& m, LaySource& src) {
+    Layered& L = *m.lay;
+    const size_t W = (size_t)m.cfg.H, V = (size_t)m.cfg.V;
+    const float ws = 1.0f / std::sqrt((float)W);
+    m.embed = up_bf16(m, src.get("embed", V * W, 1.0f, 0.f));
+    L.w.resize(L.spec.size());
+    // a one-number norm weight as a vector, so that the norm kernels of the other families apply
+    auto one_number = [&](const std::string& name, float factor) {
+        const float g = src.get(name, 1, 0.1f, 1.f)[0] * factor;
+        return up_f32(m, std::vector<float>(W, g));
+    };
+    for (size_t i = 0; i < L.spec.size(); ++i) {
+        const LayerSpec& sp = L.spec[i];
+        LayeredLayerW& w = L.w[i];
+        const std::string p = "l" + std::to_string(i) + ".";
+        w.norm1b = one_number(p + "norm1", 1.f);
+        w.side.resize(2);
+        const LayerSpec &sa = sp.side[0], &sb = sp.side[1];
+        LayeredLayerW &wa = w.side[0], &wb = w.side[1];
+        std::vector<float> in, bias;
+        {   // left: q | k | v, biases on all three
+            const size_t H = (size_t)sa.heads, G = (size_t)sa.kv_heads, d = (size_t)sa.dim, e = (size_t)sa.vdim;
+            const std::string q = p + "mix.left.";
+            wa.q_off = 0; wa.k_off = (int)(H * d); wa.v_off = wa.k_off + (int)(G * d);
+            append(in, src.get(q + "q", H * d * W, ws, 0.f)); append(bias, src.get(q + "q.b", H * d, 0.1f, 0.f));
+            append(in, src.get(q + "k", G * d * W, ws, 0.f)); append(bias, src.get(q + "k.b", G * d, 0.1f, 0.f));
+            append(in, src.get(q + "v", G * e * W, ws, 0.f)); append(bias, src.get(q + "v.b", G * e, 0.1f, 0.f));
+            wa.q_norm = up_f32(m, src.get(q + "q.norm", H * d, 0.1f, 1.f));
+            wa.k_norm = up_f32(m, src.get(q + "k.norm", G * d, 0.1f, 1.f));
+            wa.sink = up_f32(m, src.get(q + "sink", H, 1.0f, 0.f));
+            if (sa.rot.dims > 0) wa.rot_freq = up_f32(m, rot_frequencies(sa.rot, &wa.rot_mag));
+            wa.o_col = 0;
+        }
+        {   // right: q | k | v | input gate | forget gate | output gate; biases on the two recurrence gates
+            const size_t H = (size_t)sb.heads, d = (size_t)sb.dim, e = (size_t)sb.vdim;
+            const std::string q = p + "mix.right.";
+            const int base = (int)(in.size() / W);
+            wb.q_off = base; wb.k_off = wb.q_off + (int)(H * d); wb.v_off = wb.k_off + (int)(H * d); wb.i_off = wb.v_off + (int)(H * e);
+            wb.f_off = wb.i_off + (int)H; wb.g_off = wb.f_off + (int)H;
+            append(in, src.get(q + "q", H * d * W, ws, 0.f));
+            append(in, src.get(q + "k", H * d * W, ws, 0.f));
+            append(in, src.get(q + "v", H * e * W, ws, 0.f));
+            append(in, src.get(q + "i", H * W, ws, 0.f));
+            append(in, src.get(q + "f", H * W, ws, 0.f));
+            append(in, src.get(q + "g", H * e * W, ws, 0.f));
+            bias.resize((size_t)wb.i_off, 0.f);
+            append(bias, src.get(q + "i.b", H, 0.5f, 0.f));
+            append(bias, src.get(q + "f.b", H, 0.5f, 3.f));
+            wb.mix_norm = up_f32(m, src.get(q + "norm", H * e, 0.1f, 1.f));
+            wb.o_col = sa.heads * sa.vdim;
+        }
+        w.in_rows = (int)(in.size() / W);
+        w.g_off = wb.g_off;
+        bias.resize((size_t)w.in_rows, 0.f);
+        w.in_w = up_bf16(m, in);
+        w.in_b = up_f32(m, bias);
+        {   // one output projection for both mixers: the input columns are [left heads | right heads]
+            const size_t ka = (size_t)sa.heads * sa.vdim, kb = (size_t)sb.heads * sb.vdim, K = ka + kb;
+            const std::vector<float> oa = src.get(p + "mix.left.o", W * ka, 1.0f / std::sqrt((float)ka), 0.f);
+            const std::vector<float> ob = src.get(p + "mix.right.o", W * kb, 1.0f / std::sqrt((float)kb), 0.f);
+            std::vector<float> o(W * K);
+            for (size_t r = 0; r < W; ++r) {
+                std::copy(oa.begin() + (long)(r * ka), oa.begin() + (long)((r + 1) * ka), o.begin() + (long)(r * K));
+                std::copy(ob.begin() + (long)(r * kb), ob.begin() + (long)((r + 1) * kb), o.begin() + (long)(r * K + ka));
+            }
+            w.o_w = up_bf16(m, o);
+        }
+        if (sp.mlp != LMLP_NONE) {
+            w.norm2b = one_number(p + "norm2", 1.f);
+            if (sp.mlp == LMLP_MOE) build_experts(m, src, p, sp, w);
+            else {
+                const size_t ff = (size_t)sp.ff;
+                w.gate = up_bf16(m, src.get(p + "mlp.gate", ff * W, ws, 0.f));
+                w.up = up_bf16(m, src.get(p + "mlp.up", ff * W, ws, 0.f));
+                w.down = up_bf16(m, src.get(p + "mlp.down", W * ff, 1.0f / std::sqrt((float)ff), 0.f));
+            }
+        }
+    }
+    L.final_norm = one_number("final.norm", L.logit_scale);       // the factor on the logits rides on the final norm's weight
+    L.head = up_bf16(m, src.get("head", V * W, ws, 0.f));
+    m.lm_head = L.head;
+}
+
 void load_layered_from_dir(Model& m, const std::string& dir) {
     try {
         LayFileSource src(dir);
@@ -549,9 +756,8 @@ void Model::alloc_runtime_layered() {
     n_kv_layers = 0;
     kv_index.assign((size_t)cfg.L, -1);
     page_bytes = 0;
-    for (size_t i = 0; i < L.spec.size(); ++i) {
-        const LayerSpec& sp = L.spec[i];
-        LayeredLayerW& w = L.w[i];
+    // a mixer's share of the pools: cached rows of an attention, the state of a linear attention or matrix memory
+    auto place_mixer = [&](const LayerSpec& sp, LayeredLayerW& w, size_t i) {
         if (sp.mixer == LMIX_ATTN || sp.mixer == LMIX_LATENT) {
             // cached row of a token and key head: the key (latent attention: [latent | rotated key part], one head); values that
             // are not (a part of) the keys have pages of their own
@@ -562,7 +768,8 @@ void Model::alloc_runtime_layered() {
                 w.k_pool_off = o.k_pool_off; w.k_page_bytes = o.k_page_bytes; w.v_pool_off = o.v_pool_off; w.v_page_bytes = o.v_page_bytes;
                 w.kv_idx = -1;
             } else {
-                kv_index[i] = n_kv_layers++;
+                if (kv_index[i] < 0) kv_index[i] = n_kv_layers++;
+                w.kv_idx = kv_index[i];
                 w.k_page_bytes = (size_t)sp.kv_heads * page * dk * kv_esize;
                 w.k_pool_off = pool_bytes;
                 pool_bytes += (size_t)n_pages * w.k_page_bytes;
@@ -573,6 +780,21 @@ void Model::alloc_runtime_layered() {
                     w.v_pool_off = pool_bytes;
                     pool_bytes += (size_t)n_pages * w.v_page_bytes;
                     page_bytes += w.v_page_bytes;
+                }
+                if (sp.pool > 0) {             // mean rows of the position blocks that end inside a page
+                    w.pool_rows = lay_pool_rows(page, sp.pool);
+                    pool_bytes = (pool_bytes + 15) / 16 * 16;
+                    w.pk_page_bytes = (size_t)sp.kv_heads * w.pool_rows * dk * kv_esize;
+                    w.pk_pool_off = pool_bytes;
+                    pool_bytes += (size_t)n_pages * w.pk_page_bytes;
+                    page_bytes += w.pk_page_bytes;
+                    if (sp.own_v) {
+                        pool_bytes = (pool_bytes + 15) / 16 * 16;
+                        w.pv_page_bytes = (size_t)sp.kv_heads * w.pool_rows * sp.vdim * kv_esize;
+                        w.pv_pool_off = pool_bytes;
+                        pool_bytes += (size_t)n_pages * w.pv_page_bytes;
+                        page_bytes += w.pv_page_bytes;
+                    }
                 }
                 pool_bytes = (pool_bytes + 15) / 16 * 16;
             }
@@ -586,12 +808,28 @@ void Model::alloc_runtime_layered() {
                 L.max_q = std::max(L.max_q, sp.heads * (sp.dim + sp.rot_dim));
                 L.max_qa = std::max(L.max_qa, sp.heads * dk);
             }
+        } else if (sp.mixer == LMIX_MEMORY) {
+            // [H][d][e + 1] (the last column is the normaliser vector), then the running maximum [H]
+            w.st_off = st;
+            st += (size_t)sp.heads * sp.dim * (sp.vdim + 1) + (size_t)sp.heads;
+            L.max_o = std::max(L.max_o, sp.heads * (sp.vdim + 1));
+            L.max_ld = std::max(L.max_ld, sp.heads);
+            L.max_mh = std::max(L.max_mh, sp.heads);
         } else {
             w.st_off = st;
             st += (size_t)sp.heads * sp.dim * sp.vdim;
             L.max_o = std::max(L.max_o, sp.heads * sp.vdim);
             if (sp.mixer == LMIX_GLA) L.max_ld = std::max(L.max_ld, sp.heads * sp.dim);
         }
+    };
+    for (size_t i = 0; i < L.spec.size(); ++i) {
+        const LayerSpec& sp = L.spec[i];
+        LayeredLayerW& w = L.w[i];
+        if (sp.mixer == LMIX_SIDE) {
+            int ocols = 0;
+            for (size_t k = 0; k < sp.side.size(); ++k) { place_mixer(sp.side[k], w.side[k], i); ocols += sp.side[k].heads * sp.side[k].vdim; }
+            L.max_o = std::max(L.max_o, ocols);
+        } else place_mixer(sp, w, i);
         if (L.taps > 1) {
             w.c1_off = cv; cv += (size_t)(L.taps - 1) * W;
             if (sp.mlp != LMLP_NONE) { w.c2_off = cv; cv += (size_t)(L.taps - 1) * W; }
@@ -599,7 +837,12 @@ void Model::alloc_runtime_layered() {
         if (w.shift) { w.sh_off = cv; cv += W; }       // the mixer's previous input
         L.max_in = std::max(L.max_in, w.in_rows);
         if (sp.mlp != LMLP_NONE) L.max_ff = std::max(L.max_ff, sp.ff);
-        if (sp.mlp == LMLP_MOE) { L.max_top = std::max(L.max_top, sp.top); L.max_E = std::max(L.max_E, sp.experts); }
+        if (sp.mlp == LMLP_MOE) {
+            L.max_top = std::max(L.max_top, sp.top);
+            L.max_E = std::max(L.max_E, sp.experts + sp.router.identity);
+            L.max_slots = std::max(L.max_slots, sp.top + (sp.shared_ff > 0 ? 1 : 0));
+            L.max_sff = std::max(L.max_sff, sp.shared_ff);
+        }
     }
     kv_pool = (uint8_t*)dalloc<uint16_t>((pool_bytes + 1) / 2);
     free_pages.resize((size_t)n_pages);
@@ -635,15 +878,17 @@ void Model::alloc_runtime_layered() {
         L.Qa = dalloc<float>(cap * (size_t)L.max_qa);
     }
     if (L.max_ld) L.LD = dalloc<float>(cap * (size_t)L.max_ld);
+    if (L.max_mh) { L.KM = dalloc<float>(cap * (size_t)L.max_mh); L.MR = dalloc<float>(cap * (size_t)L.max_mh); }
+    if (L.max_sff) L.HS = dalloc<float>(cap * (size_t)L.max_sff);
     if (L.max_E > 1 || L.max_top > 1 || std::any_of(L.spec.begin(), L.spec.end(), [](const LayerSpec& s) { return s.mlp == LMLP_MOE; })) {
-        L.YS = dalloc<float>(cap * (size_t)L.max_top * W);
-        L.wsel = dalloc<float>(cap * (size_t)L.max_top);
+        L.YS = dalloc<float>(cap * (size_t)L.max_slots * W);
+        L.wsel = dalloc<float>(cap * (size_t)L.max_slots);
         L.sel = dalloc<int32_t>(cap * (size_t)L.max_top);
         L.srt = dalloc<int32_t>(cap * (size_t)L.max_top);
         L.off = dalloc<int32_t>((size_t)L.max_E + 1);
     }
     if (!L.f32) {
-        int max_k = std::max({(int)W, L.max_o, L.max_ff, L.max_cq}), dense_ff = 0;
+        int max_k = std::max({(int)W, L.max_o, L.max_ff, L.max_cq, L.max_sff}), dense_ff = L.max_sff;
         for (const LayerSpec& sp : L.spec) if (sp.mlp == LMLP_DENSE && sp.gated_ff) dense_ff = std::max(dense_ff, sp.ff);
         const size_t rows = (cap + 255) / 256 * 256;
         L.Abf = dalloc<uint16_t>(rows * (size_t)max_k);
@@ -652,9 +897,17 @@ void Model::alloc_runtime_layered() {
         ensure_gemm_workspace();
     }
     size_t hde = 0, hd = 0;
-    for (const LayerSpec& sp : L.spec) {
+    auto chunk_scratch = [&](const LayerSpec& sp) {
         if ((sp.mixer == LMIX_LIGHTNING || sp.mixer == LMIX_GLA) && sp.dim <= 128) hde = std::max(hde, (size_t)sp.heads * sp.dim * sp.vdim);
         if (sp.mixer == LMIX_GLA && sp.dim <= 128) hd = std::max(hd, (size_t)sp.heads * sp.dim);
+        if (sp.mixer == LMIX_MEMORY && sp.dim <= 128) {
+            hde = std::max(hde, (size_t)sp.heads * sp.dim * (sp.vdim + 1));
+            hd = std::max(hd, (size_t)sp.heads * sp.dim);
+        }
+    };
+    for (const LayerSpec& sp : L.spec) {
+        chunk_scratch(sp);
+        for (const LayerSpec& sd : sp.side) chunk_scratch(sd);
     }
     if (hde) { L.u_stride = hde; L.U = dalloc<float>((cap / LAY_LIGHT_CHUNK + (size_t)MAXB + 1) * hde); }
     if (hd) L.Dch = dalloc<float>((cap / LAY_LIGHT_CHUNK + (size_t)MAXB + 1) * hd);
@@ -703,14 +956,19 @@ void Model::layered_set_capture(bool on) {
 }
 void Model::layered_cow_page(int32_t oldp, int32_t newp) {
     Layered& L = *lay;
+    auto copy = [&](size_t off, size_t bytes) {
+        if (bytes) CM_HIP(hipMemcpyAsync(kv_pool + off + (size_t)newp * bytes, kv_pool + off + (size_t)oldp * bytes, bytes, hipMemcpyDeviceToDevice, stream));
+    };
+    auto one = [&](const LayeredLayerW& w) {
+        if (w.kv_idx < 0) return;
+        copy(w.k_pool_off, w.k_page_bytes);
+        copy(w.v_pool_off, w.v_page_bytes);
+        copy(w.pk_pool_off, w.pk_page_bytes);
+        copy(w.pv_pool_off, w.pv_page_bytes);
+    };
     for (size_t i = 0; i < L.w.size(); ++i) {
-        const LayeredLayerW& w = L.w[i];
-        if (w.kv_idx < 0) continue;
-        CM_HIP(hipMemcpyAsync(kv_pool + w.k_pool_off + (size_t)newp * w.k_page_bytes, kv_pool + w.k_pool_off + (size_t)oldp * w.k_page_bytes,
-                              w.k_page_bytes, hipMemcpyDeviceToDevice, stream));
-        if (w.v_page_bytes)
-            CM_HIP(hipMemcpyAsync(kv_pool + w.v_pool_off + (size_t)newp * w.v_page_bytes, kv_pool + w.v_pool_off + (size_t)oldp * w.v_page_bytes,
-                                  w.v_page_bytes, hipMemcpyDeviceToDevice, stream));
+        one(L.w[i]);
+        for (const LayeredLayerW& sd : L.w[i].side) one(sd);
     }
 }
 
@@ -827,8 +1085,8 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
         const LaySegDev* d_segs = (const LaySegDev*)(L.d_tab + o_segs);
         const int32_t* d_bt = L.d_tab + o_bt;
 
-        if (W % 4 == 0) launch_embed_rows(embed, d_ids, L.X, T, W, V, s);
-        else launch_lay_embed_rows(embed, d_ids, L.X, T, W, V, s);
+        if (W % 4 == 0 && L.embed_scale == 1.f) launch_embed_rows(embed, d_ids, L.X, T, W, V, s);
+        else launch_lay_embed_rows(embed, d_ids, L.X, T, W, V, s, L.embed_scale);
         // the residual update of a finished sublayer waits for the next norm: decode steps run both in one launch
         struct { const float* y = nullptr; const float* w = nullptr; const float* wsel = nullptr; int top = 0; } pend;
         auto flush_post = [&]() {
@@ -857,10 +1115,15 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
             launch_lay_canon_tail(L.Hn, conv_pool, conv_slot_elems, coff, d_segs, nseg, W, L.taps, s);
         };
         // softmax attention of one layer over the pages: queries at qsrc[row ldq + q_off + head dk], output [T][H ev] into L.O
-        auto run_attention = [&](const LayerSpec& sp, const LayeredLayerW& w, const float* qsrc, int ldq, int q_off, int g_off, int dk, int ev) {
+        auto run_attention = [&](const LayerSpec& sp, const LayeredLayerW& w, const float* qsrc, int ldq, int q_off, int g_off, int dk, int ev,
+                                 float* out = nullptr, int ldo = 0, float out_scale = 1.f) {
             LAttnArgs a;
             a.proj = qsrc; a.ldp = ldq; a.q_off = q_off; a.g_off = g_off;
-            a.out = L.O; a.ldo = sp.heads * ev;
+            a.out = out ? out : L.O; a.ldo = out ? ldo : sp.heads * ev; a.out_scale = out_scale;
+            if (sp.pool > 0) {
+                a.pool = sp.pool; a.pool_rows = w.pool_rows; a.pk_pool = kv_pool + w.pk_pool_off;
+                a.pv_pool = w.pv_page_bytes ? kv_pool + w.pv_pool_off : nullptr;
+            }
             a.kpool = kv_pool + w.k_pool_off; a.bt = d_bt; a.segs = d_segs;
             a.vpool = w.v_page_bytes ? kv_pool + w.v_pool_off : nullptr; a.e = ev;
             const auto& tl = tiles[sp.heads / sp.kv_heads];
@@ -871,6 +1134,7 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
             {   // few query tiles and many visible keys (decode steps): share a tile's keys among blocks
                 long long seen = std::min<long long>(max_len, sp.win + sp.keep);
                 if (sp.chunk > 0) seen = std::min(seen, sp.chunk);
+                if (sp.pool > 0) seen = std::min<long long>(max_len, sp.win + max_len / sp.pool);
                 const int kt = lay_attn_key_tile(dk, ev, a.vpool != nullptr);
                 const int key_tiles = (int)((seen + kt - 1) / kt), blocks = std::max(1, a.ntiles * sp.kv_heads);
                 a.nsplit = std::max(1, std::min({32, key_tiles, 256 / blocks, Layered::ATT_PARTS / blocks}));
@@ -884,14 +1148,20 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                 launch_lay_attn(a, kv_mode, s);
         };
         // lightning / gated linear attention of one layer: raw head outputs into L.O
-        auto run_linear = [&](const LayerSpec& sp, const LayeredLayerW& w, const float* ldec) {
+        // ldp: width of the projection rows in L.P; kmul != null: the matrix-memory form (one decay and one key factor per head and
+        // token, a constant 1 as last value column, raw outputs [T][H (e + 1)] into L.O2)
+        auto run_linear = [&](const LayerSpec& sp, const LayeredLayerW& w, const float* ldec, int ldp, const float* kmul = nullptr) {
             LLightArgs a;
-            a.proj = L.P; a.ldp = w.in_rows; a.q_off = w.q_off; a.k_off = w.k_off; a.v_off = w.v_off;
+            a.proj = L.P; a.ldp = ldp; a.q_off = w.q_off; a.k_off = w.k_off; a.v_off = w.v_off;
             a.out = L.O; a.ldo = sp.heads * sp.vdim;
             a.state_pool = state_pool; a.slot_stride = state_slot_elems; a.st_off = w.st_off;
             a.segs = d_segs; a.nseg = nseg; a.decay = w.decay; a.H = sp.heads; a.d = sp.dim; a.e = sp.vdim;
             a.all_single = all_decode;
             if (ldec) { a.ldec = ldec; a.ldd = sp.heads * sp.dim; a.qscale = 1.0f / std::sqrt((float)sp.dim); a.D = L.Dch; }
+            if (kmul) {
+                a.head_decay = true; a.kmul = kmul; a.ones_col = true; a.ldd = sp.heads;
+                a.e = sp.vdim + 1; a.out = L.O2; a.ldo = sp.heads * (sp.vdim + 1);
+            }
             if (L.U && max_n > LAY_LIGHT_CHUNK && sp.dim <= 128) {       // a long portion in the pass: parallel over chunks
                 a.U = L.U; a.chunks = (const int2*)(L.d_tab + o_chunks); a.nchunks = nchunks;
             }
@@ -959,7 +1229,7 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                     gd.A = L.P + w.a_off; gd.lda = w.in_rows; gd.W = w.a2; gd.bias = w.a2_b; gd.C = L.LD; gd.ldc = H * sp.dim;
                     gd.M = T; gd.N = H * sp.dim; gd.K = sp.a_rank; gd.act = LACT_LOGSIG; gd.act_split = gd.N; gd.act_param = 1.0f / sp.tau;
                     lay_gemm(*this, L, gd, 1, s);
-                    run_linear(sp, w, L.LD);
+                    run_linear(sp, w, L.LD, w.in_rows);
                     launch_lay_rms_gate(L.O, L.P + w.g_off, w.in_rows, w.mix_norm, L.O2, T, H * ev, cfg.eps, s, ev, true);
                     oa = L.O2;
                 }
@@ -980,6 +1250,89 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                     launch_lay_add_rows(L.X, par_y1, par_y2, (size_t)T * W, s);
                     par_y1 = par_y2 = nullptr;
                 }
+            } else if (L.post_only) {
+                // ---- the sublayers read the residual itself; x += g * unit(sublayer(x)).  All mixers of the layer share one input
+                // projection and one output projection (their heads side by side in its input, each times its scale)
+                flush_post();
+                LGemmArgs g;
+                g.A = L.X; g.lda = W; g.W = w.in_w; g.bias = w.in_b; g.C = L.P; g.ldc = w.in_rows; g.M = T; g.N = w.in_rows; g.K = W;
+                g.act_split = w.g_off; g.act = LACT_NONE; g.act2 = LACT_SIGMOID;
+                lay_gemm(*this, L, g, 1, s);
+                int ocols = 0;
+                for (const LayerSpec& sd : sp.side) ocols += sd.heads * sd.vdim;
+                for (size_t k = 0; k < sp.side.size(); ++k) {
+                    const LayerSpec& sd = sp.side[k];
+                    const LayeredLayerW& sw = w.side[k];
+                    const int H = sd.heads, G = sd.kv_heads, d = sd.dim, e = sd.vdim;
+                    if (sd.mixer == LMIX_ATTN) {
+                        if (sd.qk_norm) {
+                            launch_lay_rms_cols(L.P, w.in_rows, sw.q_off, H * d, sw.q_norm, L.P + sw.q_off, w.in_rows, T, cfg.eps, s);
+                            launch_lay_rms_cols(L.P, w.in_rows, sw.k_off, G * d, sw.k_norm, L.P + sw.k_off, w.in_rows, T, cfg.eps, s);
+                        }
+                        if (sd.rot.dims > 0) {
+                            launch_lay_rope(L.P + sw.q_off, w.in_rows, d, L.P + sw.q_off, w.in_rows, d, H, d, sd.rot.dims, sw.rot_freq, sw.rot_mag,
+                                            d_segs, d_rowseg, T, s, sd.rot.half);
+                            launch_lay_rope(L.P + sw.k_off, w.in_rows, d, L.P + sw.k_off, w.in_rows, d, G, d, sd.rot.dims, sw.rot_freq, sw.rot_mag,
+                                            d_segs, d_rowseg, T, s, sd.rot.half);
+                        }
+                        launch_lay_k_append(L.P, w.in_rows, sw.k_off, kv_pool + sw.k_pool_off, kv_mode, d_bt, d_segs, d_rowseg, T, G, d, page, s);
+                        launch_lay_k_append(L.P, w.in_rows, sw.v_off, kv_pool + sw.v_pool_off, kv_mode, d_bt, d_segs, d_rowseg, T, G, e, page, s);
+                        if (sd.pool > 0) {
+                            launch_lay_pool_append(kv_pool + sw.k_pool_off, kv_pool + sw.pk_pool_off, kv_mode, d_bt, d_segs, d_rowseg, T, G, d, page,
+                                                   (int)sd.pool, sw.pool_rows, s);
+                            launch_lay_pool_append(kv_pool + sw.v_pool_off, kv_pool + sw.pv_pool_off, kv_mode, d_bt, d_segs, d_rowseg, T, G, e, page,
+                                                   (int)sd.pool, sw.pool_rows, s);
+                        }
+                        run_attention(sd, sw, L.P, w.in_rows, sw.q_off, 0, d, e, L.O + sw.o_col, ocols, sd.side_scale);
+                    } else if (sd.mixer == LMIX_MEMORY) {
+                        launch_lay_memory_gates(L.P, w.in_rows, sw.i_off, sw.f_off, sd.gate_cap, L.LD, L.KM, L.MR, state_pool, state_slot_elems,
+                                                sw.st_off + (size_t)H * d * (e + 1), d_segs, nseg, H, s);
+                        run_linear(sd, sw, L.LD, w.in_rows, L.KM);
+                        launch_lay_memory_out(L.O2, L.MR, L.P + sw.g_off, w.in_rows, sw.mix_norm, L.O + sw.o_col, ocols, T, H, e, cfg.eps,
+                                              sd.side_scale, s);
+                    } else throw CmError(CM_ERR_UNSUPPORTED, "side mixer kind");
+                }
+                LGemmArgs go;
+                go.A = L.O; go.lda = ocols; go.W = w.o_w; go.C = L.Y; go.ldc = W; go.M = T; go.N = W; go.K = ocols;
+                lay_gemm(*this, L, go, 1, s);
+                post_norm(L.Y, w.norm1b, nullptr, 0);
+                if (sp.mlp == LMLP_DENSE) {
+                    flush_post();
+                    LGemmArgs gu;
+                    gu.A = L.X; gu.lda = W; gu.W = w.gate; gu.W2 = w.up; gu.C = L.HH; gu.ldc = sp.ff; gu.M = T; gu.N = sp.ff; gu.K = W;
+                    gu.act = sp.ff_act;
+                    lay_gemm(*this, L, gu, 1, s);
+                    LGemmArgs dn;
+                    dn.A = L.HH; dn.lda = sp.ff; dn.W = w.down; dn.C = L.Y; dn.ldc = W; dn.M = T; dn.N = W; dn.K = sp.ff;
+                    lay_gemm(*this, L, dn, 1, s);
+                    post_norm(L.Y, w.norm2b, nullptr, 0);
+                } else if (sp.mlp == LMLP_MOE) {
+                    flush_post();
+                    const int outs = sp.experts + sp.router.identity, slots = sp.top + (sp.shared_ff > 0 ? 1 : 0);
+                    launch_lay_router(L.X, w.router, L.sel, L.wsel, T, W, outs, sp.top, s, &sp.router, w.correction, slots);
+                    launch_lay_moe_plan(L.sel, L.off, L.srt, T * sp.top, outs, s, sp.top, slots);
+                    LGemmArgs gu;
+                    gu.A = L.X; gu.lda = W; gu.a_idx = L.srt; gu.a_div = slots;
+                    gu.W = w.gate; gu.W2 = w.up; gu.w_stride = (size_t)sp.ff * W;
+                    gu.C = L.HH; gu.ldc = sp.ff; gu.M = T; gu.N = sp.ff; gu.K = W; gu.grp_off = L.off; gu.act = LACT_SILU;
+                    lay_gemm(*this, L, gu, sp.experts, s);
+                    LGemmArgs dn;
+                    dn.A = L.HH; dn.lda = sp.ff; dn.W = w.down; dn.w_stride = (size_t)W * sp.ff;
+                    dn.C = L.YS; dn.ldc = W; dn.c_idx = L.srt; dn.M = T; dn.N = W; dn.K = sp.ff; dn.grp_off = L.off;
+                    lay_gemm(*this, L, dn, sp.experts, s);
+                    if (sp.router.identity > 0) launch_lay_moe_identity(L.sel, L.X, L.YS, T, W, sp.top, slots, sp.experts, s);
+                    if (sp.shared_ff > 0) {        // the expert every token uses: row `top` of the token's rows, weight 1
+                        LGemmArgs su;
+                        su.A = L.X; su.lda = W; su.W = w.sh_gate; su.W2 = w.sh_up; su.C = L.HS; su.ldc = sp.shared_ff; su.M = T; su.N = sp.shared_ff;
+                        su.K = W; su.act = LACT_SILU;
+                        lay_gemm(*this, L, su, 1, s);
+                        LGemmArgs sdn;
+                        sdn.A = L.HS; sdn.lda = sp.shared_ff; sdn.W = w.sh_down; sdn.C = L.YS + (size_t)sp.top * W; sdn.ldc = slots * W; sdn.M = T;
+                        sdn.N = W; sdn.K = sp.shared_ff;
+                        lay_gemm(*this, L, sdn, 1, s);
+                    }
+                    post_norm(L.YS, w.norm2b, L.wsel, slots);
+                }
             } else {
             norm_canon(w.norm1, w.canon1, w.c1_off);
             LGemmArgs g;
@@ -994,7 +1347,7 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                 run_attention(sp, w, L.P, w.in_rows, w.q_off, w.g_off, sp.dim, sp.dim);
                 on = sp.heads * sp.dim; oa = L.O;
             } else {
-                run_linear(sp, w, nullptr);
+                run_linear(sp, w, nullptr, w.in_rows);
                 on = sp.heads * sp.vdim;
                 launch_lay_rms_gate(L.O, L.P + w.g_off, w.in_rows, w.mix_norm, L.O2, T, on, cfg.eps, s);
                 oa = L.O2;
