@@ -146,7 +146,7 @@ def relaunch_under_torchrun(n: int) -> int:
 
 
 def korupel_leg(args, names=None, prompt_lens=None, label="korupel"):
-    """--korupel / --mononex: prompt and decode throughput of a layer-list decoder (Korupel, Mononex; crane_amd/csrc/model_layered.cpp)
+    """--korupel / --mononex / --gibipel: prompt and decode throughput of a layer-list decoder (Korupel, Mononex, Gibipel; crane_amd/csrc/model_layered.cpp)
     at the widths of a real model, random weights, beside the closest family of the library at equal size: the Qwen3.5 hybrid
     (linear attention 3 : 1 softmax attention, same width / ff / layers / vocabulary).  One JSON line; the default workload of this
     script is not touched."""
@@ -250,11 +250,16 @@ def main():
     ap.add_argument("--mononex", default=None, metavar="CONFIGS", help="comma-separated registry configs (e.g. "
                     "mononex-1b,korupel-1b,qwen3.5-0.8b): prompt and decode throughput of each instead of the headline workload")
     ap.add_argument("--mononex-prompts", default="512,2048", help="prompt lengths of --mononex")
+    ap.add_argument("--gibipel", default=None, metavar="CONFIGS", help="comma-separated registry configs (e.g. "
+                    "gibipel-1b,korupel-1b-moe,qwen3.5-0.8b): prompt and decode throughput of each instead of the headline workload")
+    ap.add_argument("--gibipel-prompts", default="512,2048", help="prompt lengths of --gibipel")
     args = ap.parse_args()
     if args.korupel:
         sys.exit(korupel_leg(args))
     if args.mononex:
         sys.exit(korupel_leg(args, args.mononex, args.mononex_prompts, "mononex"))
+    if args.gibipel:
+        sys.exit(korupel_leg(args, args.gibipel, args.gibipel_prompts, "gibipel"))
 
     if args.tp_inprocess:      # ranks that share a device need one hardware queue per rank stream: before the HIP runtime starts
         os.environ.setdefault("GPU_MAX_HW_QUEUES", "16")

@@ -226,6 +226,50 @@ CONFIGS.update({
 })
 
 
+# ---- layer-list decoders: Gibipel ------------------------------------------------------------------------------------------
+def gibipel_config(vocab: int, width: int, n_layers: int, heads: int, kv_heads: int, dim: int, vdim: int, window: int, pool: int,
+                   mem_heads: int, mem_dim: int, mem_vdim: int, experts: int, top: int, expert_ff: int, identity: int = 0,
+                   groups: int = 1, keep_groups: int = 1, shared_ff: int = 0, rot_dims: "int | None" = None, rot_base: float = 10000.0,
+                   scaling: "dict | None" = None, left_scale: float = 1.0, right_scale: float = 1.0, gate_cap: float = 15.0,
+                   embed_scale: float = 1.0, logit_scale: float = 1.0, eps: float = 1e-5, no_ff: "tuple | list" = ()) -> dict:
+    """Every layer holds both mixers side by side: window attention that sees the blocks of `pool` positions in front of its
+    window through their mean key / value, and a matrix memory; a mixture-of-experts feed-forward (layers in `no_ff`: none)."""
+    layers = []
+    for i in range(n_layers):
+        rot = dict(base=rot_base, dims=dim if rot_dims is None else rot_dims)
+        if scaling:
+            rot["scaling"] = dict(scaling)
+        left = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=dim ** -0.5, mask=dict(size=window, pool=pool), rot=rot)
+        right = dict(heads=mem_heads, dim=mem_dim, vdim=mem_vdim, gate_cap=gate_cap)
+        mlp = None
+        if i not in no_ff:
+            mlp = dict(kind="moe", expert=dict(ff=expert_ff),
+                       router=dict(experts=experts, top=top, identity=identity, groups=dict(count=groups, keep=keep_groups)))
+            if shared_ff:
+                mlp["shared"] = dict(ff=shared_ff)
+        layers.append(dict(type="parallel", mixer=dict(left=left, right=right, left_scale=left_scale, right_scale=right_scale), mlp=mlp))
+    return dict(architecture="Gibipel", vocab=vocab, width=width, norm=dict(eps=eps), embedding=dict(scale=embed_scale),
+                logit_scale=logit_scale, layers=layers)
+
+
+_BANDS = dict(factor=8.0, low=1.0, high=4.0, original=8192)
+CONFIGS.update({
+    "tiny-gibipel": gibipel_config(320, 128, 3, heads=4, kv_heads=2, dim=32, vdim=16, window=20, pool=6, mem_heads=2, mem_dim=16,
+                                   mem_vdim=24, experts=6, top=2, expert_ff=48, identity=2, groups=2, keep_groups=1, shared_ff=64,
+                                   rot_dims=16, scaling=dict(factor=4.0, low=1.0, high=4.0, original=64), left_scale=0.7,
+                                   right_scale=1.2, embed_scale=4.0, logit_scale=0.5, no_ff=(1,)),
+    # the widths of the Qwen3.5-0.8B text decoder and of korupel-1b-moe (1024 wide, 24 layers, vocabulary 248 320, 8 query / 2 key
+    # heads of 128): window 1024 and blocks of 64, 8 memory heads of 64 x 128, 14 experts + 2 identity experts in 2 groups, 4 per
+    # token, of 768, and a shared expert of 512 (3584 active inner columns, as the dense models)
+    "gibipel-1b": gibipel_config(248320, 1024, 24, heads=8, kv_heads=2, dim=128, vdim=128, window=1024, pool=64, mem_heads=8, mem_dim=64,
+                                 mem_vdim=128, experts=14, top=4, expert_ff=768, identity=2, groups=2, keep_groups=1, shared_ff=512,
+                                 scaling=_BANDS, rot_base=500000.0),
+    "gibipel-1b-4l": gibipel_config(32768, 1024, 4, heads=8, kv_heads=2, dim=128, vdim=128, window=1024, pool=64, mem_heads=8, mem_dim=64,
+                                    mem_vdim=128, experts=14, top=4, expert_ff=768, identity=2, groups=2, keep_groups=1, shared_ff=512,
+                                    scaling=_BANDS, rot_base=500000.0),
+})
+
+
 def get_config(name: str) -> dict:
     if name not in CONFIGS:
         raise KeyError(f"unknown config {name!r}; have {sorted(CONFIGS)}")

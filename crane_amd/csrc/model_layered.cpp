@@ -1431,26 +1431,39 @@ uint64_t Model::layered_decode_bytes(size_t ctx) const {
     const Layered& L = *lay;
     const uint64_t W = (uint64_t)cfg.H;
     uint64_t b = 2ull * (uint64_t)cfg.V * W + 2ull * W;       // head + one embedding row
-    for (size_t i = 0; i < L.spec.size(); ++i) {
-        const LayerSpec& sp = L.spec[i];
-        b += 2ull * (uint64_t)L.w[i].in_rows * W;
+    // cached rows or state that one decode token of a mixer reads (and writes), and its own matrices besides the input projection
+    auto mixer_bytes = [&](const LayerSpec& sp) {
+        uint64_t n = 0;
         if (sp.mixer == LMIX_ATTN || sp.mixer == LMIX_LATENT) {
             const uint64_t H = (uint64_t)sp.heads;
             uint64_t row = (uint64_t)sp.kv_heads * sp.dim + (sp.own_v ? (uint64_t)sp.kv_heads * sp.vdim : 0);      // cached elements per token
             if (sp.mixer == LMIX_LATENT) {
                 row = (uint64_t)sp.kv_rank + sp.rot_dim;
-                b += 2ull * (H * (sp.dim + sp.rot_dim) * sp.q_rank + H * sp.dim * sp.kv_rank + H * sp.vdim * sp.kv_rank);
+                n += 2ull * (H * (sp.dim + sp.rot_dim) * sp.q_rank + H * sp.dim * sp.kv_rank + H * sp.vdim * sp.kv_rank);
             }
-            b += 2ull * W * H * sp.vdim;
+            n += 2ull * W * H * sp.vdim;
             uint64_t seen = std::min<uint64_t>(ctx, (uint64_t)std::min<long long>(sp.win, 1ll << 40) + (uint64_t)sp.keep);
             if (sp.chunk > 0) seen = std::min<uint64_t>(seen, (uint64_t)sp.chunk);
-            b += seen * row * kv_esize;
+            if (sp.pool > 0 && ctx > seen) seen += (ctx - seen) / (uint64_t)sp.pool;       // one mean row per block in front of the window
+            n += seen * row * kv_esize;
+        } else if (sp.mixer == LMIX_MEMORY) {
+            n += 2ull * W * sp.heads * sp.vdim + 8ull * sp.heads * sp.dim * (sp.vdim + 1);
         } else {
-            b += 2ull * W * sp.heads * sp.vdim + 8ull * sp.heads * sp.dim * sp.vdim;    // state read + write
-            if (sp.mixer == LMIX_GLA) b += 2ull * sp.heads * sp.dim * sp.a_rank;
+            n += 2ull * W * sp.heads * sp.vdim + 8ull * sp.heads * sp.dim * sp.vdim;    // state read + write
+            if (sp.mixer == LMIX_GLA) n += 2ull * sp.heads * sp.dim * sp.a_rank;
         }
+        return n;
+    };
+    for (size_t i = 0; i < L.spec.size(); ++i) {
+        const LayerSpec& sp = L.spec[i];
+        b += 2ull * (uint64_t)L.w[i].in_rows * W;
+        if (sp.mixer == LMIX_SIDE) { for (const LayerSpec& sd : sp.side) b += mixer_bytes(sd); }
+        else b += mixer_bytes(sp);
         if (sp.mlp == LMLP_DENSE) b += (sp.gated_ff ? 6ull : 4ull) * W * sp.ff;
-        else if (sp.mlp == LMLP_MOE) b += 6ull * W * sp.ff * sp.top + 2ull * W * sp.experts;
+        else if (sp.mlp == LMLP_MOE) {
+            const uint64_t real = (uint64_t)std::min(sp.top, sp.experts);
+            b += 6ull * W * sp.ff * real + 2ull * W * (sp.experts + sp.router.identity) + 6ull * W * sp.shared_ff;
+        }
     }
     return b;
 }

@@ -82,7 +82,9 @@ def visible_tokens(i, window):
 
 
 def visible_blocks(i, window, pool):
-    """Blocks [bP, bP + P) that lie wholly in front of position i's window."""
+    """Blocks [bP, bP + P) that lie wholly in front of position i's window (no pooling: none)."""
+    if not pool:
+        return []
     return [b for b in range((i + 1) // pool + 1) if b * pool + pool - 1 <= i - window]
 
 
@@ -115,7 +117,7 @@ def pooled_window_attention(q, k, v, sink, scale, window, pool):
     T, H, _ = q.shape
     G, e = k.shape[1], v.shape[2]
     out = np.zeros((T, H, e))
-    nb = T // pool
+    nb = T // pool if pool else 0
     kb = k[:nb * pool].reshape(nb, pool, G, -1).mean(1) if nb else np.zeros((0,) + k.shape[1:])
     vb = v[:nb * pool].reshape(nb, pool, G, -1).mean(1) if nb else np.zeros((0,) + v.shape[1:])
     for hd in range(H):
@@ -135,7 +137,7 @@ def left_mixer(h, P, pre, mx, eps):
     T = h.shape[0]
     q = left_queries(h, P, pre, mx, eps)
     k, v = left_keys_values(h, P, pre, mx, eps)
-    o = pooled_window_attention(q, k, v, P[pre + "sink"], mx["scale"], mx["mask"]["size"], mx["mask"]["pool"])
+    o = pooled_window_attention(q, k, v, P[pre + "sink"], mx["scale"], mx["mask"]["size"], mx["mask"].get("pool", 0))
     return o.reshape(T, -1) @ P[pre + "o"].T
 
 
