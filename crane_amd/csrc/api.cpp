@@ -576,6 +576,7 @@ int cm_debug_set(cm_model* h, const char* key, int64_t value) {
         if (k == "lay_capture") mm.layered_set_capture(value != 0);
         else if (k == "lay_shared_gemm") mm.layered_set_shared_gemm(value != 0);
         else if (k == "lay_attn_mfma") mm.layered_set_attn_mfma(value != 0);
+        else if (k == "lay_fused_prep") mm.layered_set_fused_prep(value != 0);
         else if (k == "no_prefill") mm.no_prefill = value != 0;
         else if (k == "quant_prefill") mm.quant_prefill = value != 0;
         else if (k == "prefill_q8") {       // before the first prompt pass of the handle: 0 = prompts over Q8_0-layout weights on the dequantised-to-bf16 GEMMs

@@ -743,6 +743,7 @@ __global__ __launch_bounds__(256) void lay_act_cols_kernel(float* __restrict__ C
 }
 void launch_lay_act_cols(float* C, int ldc, int M, int N, int act, int act2, int split, hipStream_t s, float param) {
     if (M <= 0 || ((act == LACT_NONE || split <= 0) && (act2 == LACT_NONE || split >= N))) return;
+    if (act == LACT_NONE && split > 0) { C += split; N -= split; split = 0; }       // the columns in front stay as they are: not swept
     hipLaunchKernelGGL(lay_act_cols_kernel, dim3((unsigned)M, (unsigned)((N + 255) / 256)), dim3(256), 0, s, C, ldc, N, act, act2, split, param);
 }
 // out = act(g) * u
@@ -840,36 +841,123 @@ __device__ __forceinline__ LaRow la_row(const LAttnArgs& a, const LaySegDev& sg,
     return r;
 }
 
-// one block per row of the pass; a row whose position closes a block of `pool` positions writes the block's mean row (f32 sum in
-// position order, then one rounding into the cache's format)
+// one block per row of the pass (blockIdx.y: keys / values); a row whose position closes a block of `pool` positions writes the block's
+// mean row (f32 sum in position order, then one rounding into the cache's format)
 template <int KVT>
-__global__ __launch_bounds__(256) void lay_pool_append_kernel(const void* __restrict__ kpool, void* __restrict__ pk_pool,
+__global__ __launch_bounds__(256) void lay_pool_append_kernel(const void* __restrict__ kpool, void* __restrict__ pk_pool, int d,
+                                                              const void* __restrict__ vpool, void* __restrict__ pv_pool, int e,
                                                               const int32_t* __restrict__ bt, const LaySegDev* __restrict__ segs,
-                                                              const int32_t* __restrict__ rowseg, int G, int d, int page, int pool, int pool_rows) {
+                                                              const int32_t* __restrict__ rowseg, int G, int page, int pool, int pool_rows) {
     const int r = blockIdx.x;
     const LaySegDev sg = segs[rowseg[r]];
     const int pos = sg.start_pos + (r - sg.row0);
     if ((pos + 1) % pool != 0) return;
+    const void* src = blockIdx.y ? vpool : kpool;
+    void* dstp = blockIdx.y ? pv_pool : pk_pool;
+    const int n = blockIdx.y ? e : d;
     const int b = (pos + 1) / pool - 1, lpg = pos / page;
     const int idx = b - (int)(((long long)lpg * page) / pool);
     const float inv = 1.f / (float)pool;
-    for (int i = threadIdx.x; i < G * d; i += 256) {
-        const int g = i / d, c = i - g * d;
+    for (int i = threadIdx.x; i < G * n; i += 256) {
+        const int g = i / n, c = i - g * n;
         float sum = 0.f;
+#pragma unroll 8
         for (int j = b * pool; j <= pos; ++j) {
-            const size_t src = (((size_t)bt[sg.bt_off + j / page] * G + g) * page + (size_t)(j % page)) * d + c;
-            sum += KVT == KV_F32 ? ((const float*)kpool)[src] : bf16_to_f32(((const uint16_t*)kpool)[src]);
+            const size_t at = (((size_t)bt[sg.bt_off + j / page] * G + g) * page + (size_t)(j % page)) * n + c;
+            sum += KVT == KV_F32 ? ((const float*)src)[at] : bf16_to_f32(((const uint16_t*)src)[at]);
         }
-        const size_t dst = (((size_t)bt[sg.bt_off + lpg] * G + g) * pool_rows + idx) * d + c;
-        if (KVT == KV_F32) ((float*)pk_pool)[dst] = sum * inv;
-        else ((uint16_t*)pk_pool)[dst] = f32_to_bf16(sum * inv);
+        const size_t dst = (((size_t)bt[sg.bt_off + lpg] * G + g) * pool_rows + idx) * n + c;
+        if (KVT == KV_F32) ((float*)dstp)[dst] = sum * inv;
+        else ((uint16_t*)dstp)[dst] = f32_to_bf16(sum * inv);
     }
 }
-void launch_lay_pool_append(const void* kpool, void* pk_pool, int kvt, const int32_t* bt, const LaySegDev* segs, const int32_t* rowseg, int T,
-                            int G, int d, int page, int pool, int pool_rows, hipStream_t s) {
+void launch_lay_pool_append(const void* kpool, void* pk_pool, int d, const void* vpool, void* pv_pool, int e, int kvt, const int32_t* bt,
+                            const LaySegDev* segs, const int32_t* rowseg, int T, int G, int page, int pool, int pool_rows, hipStream_t s) {
     if (T <= 0 || pool <= 0) return;
-    if (kvt == KV_F32) hipLaunchKernelGGL(lay_pool_append_kernel<KV_F32>, dim3((unsigned)T), dim3(256), 0, s, kpool, pk_pool, bt, segs, rowseg, G, d, page, pool, pool_rows);
-    else hipLaunchKernelGGL(lay_pool_append_kernel<KV_BF16>, dim3((unsigned)T), dim3(256), 0, s, kpool, pk_pool, bt, segs, rowseg, G, d, page, pool, pool_rows);
+    const dim3 grid((unsigned)T, vpool ? 2u : 1u);
+    if (kvt == KV_F32) hipLaunchKernelGGL(lay_pool_append_kernel<KV_F32>, grid, dim3(256), 0, s, kpool, pk_pool, d, vpool, pv_pool, e, bt, segs, rowseg, G, page, pool, pool_rows);
+    else hipLaunchKernelGGL(lay_pool_append_kernel<KV_BF16>, grid, dim3(256), 0, s, kpool, pk_pool, d, vpool, pv_pool, e, bt, segs, rowseg, G, page, pool, pool_rows);
+}
+
+// Queries and keys on their way into attention, one block per row of the pass: RMS norm over all query heads at once and over all
+// key heads at once (weights qn / kn; null: none), rotation by position (pairs (2i, 2i + 1) or (i, i + dims / 2) of the first dims
+// elements of each head), q back in place, the key row -- and the value row at v_off, when vpool is given -- into the sequence's pages.
+struct LQkPrepArgs {
+    float* proj; int ldp, q_off, k_off, v_off;
+    int H, G, d, e;
+    const float *qn, *kn; float eps;
+    int dims, half; const float* freq; float mag;
+    void *kpool, *vpool;
+    const int32_t* bt; const LaySegDev* segs; const int32_t* rowseg; int page;
+};
+template <int KVT>
+__global__ __launch_bounds__(256) void lay_qk_prep_kernel(LQkPrepArgs a) {
+    __shared__ float red[4];
+    const int r = blockIdx.x, tid = threadIdx.x;
+    const LaySegDev sg = a.segs[a.rowseg[r]];
+    const int pos = sg.start_pos + (r - sg.row0);
+    float* q = a.proj + (size_t)r * a.ldp + a.q_off;
+    float* k = a.proj + (size_t)r * a.ldp + a.k_off;
+    const int nq = a.H * a.d, nk = a.G * a.d;
+    float rq = 1.f, rk = 1.f;
+    if (a.qn) {
+        float ss = 0.f;
+        for (int i = tid; i < nq; i += 256) { const float v = q[i]; ss += v * v; }
+        rq = 1.f / sqrtf(block_sum(ss, red) / (float)nq + a.eps);
+    }
+    if (a.kn) {
+        float ss = 0.f;
+        for (int i = tid; i < nk; i += 256) { const float v = k[i]; ss += v * v; }
+        rk = 1.f / sqrtf(block_sum(ss, red) / (float)nk + a.eps);
+    }
+    const int pg = a.bt[sg.bt_off + pos / a.page];
+    const size_t prow = (size_t)pg * a.G * a.page + (size_t)(pos % a.page);       // + g * page: the cached row of key head g
+    // a thread owns both elements of a pair (or one element past the rotated part)
+    const int hd = a.dims / 2, per = hd + (a.d - a.dims);
+    const float fpos = (float)pos;
+    for (int idx = tid; idx < (a.H + a.G) * per; idx += 256) {
+        const int v = idx / per, i = idx - v * per;
+        const bool isq = v < a.H;
+        const int hh = isq ? v : v - a.H;
+        float* x = (isq ? q : k) + hh * a.d;
+        const float* w = isq ? a.qn : a.kn;
+        const float rs = isq ? rq : rk;
+        int i0, i1 = -1;
+        if (i < hd) { i0 = a.half ? i : 2 * i; i1 = a.half ? i + hd : 2 * i + 1; }
+        else i0 = a.dims + (i - hd);
+        float x0 = x[i0] * rs, x1 = i1 >= 0 ? x[i1] * rs : 0.f;
+        if (w) { x0 *= w[hh * a.d + i0]; if (i1 >= 0) x1 *= w[hh * a.d + i1]; }
+        if (i1 >= 0) {
+            float sn, cs;
+            sincosf(fpos * a.freq[i], &sn, &cs);
+            sn *= a.mag; cs *= a.mag;
+            const float y0 = x0 * cs - x1 * sn, y1 = x1 * cs + x0 * sn;
+            x0 = y0; x1 = y1;
+        }
+        if (isq) { x[i0] = x0; if (i1 >= 0) x[i1] = x1; }
+        else {
+            const size_t dst = (prow + (size_t)hh * a.page) * a.d;
+            if (KVT == KV_F32) { ((float*)a.kpool)[dst + i0] = x0; if (i1 >= 0) ((float*)a.kpool)[dst + i1] = x1; }
+            else { ((uint16_t*)a.kpool)[dst + i0] = f32_to_bf16(x0); if (i1 >= 0) ((uint16_t*)a.kpool)[dst + i1] = f32_to_bf16(x1); }
+        }
+    }
+    if (a.vpool) {
+        const float* vv = a.proj + (size_t)r * a.ldp + a.v_off;
+        for (int i = tid; i < a.G * a.e; i += 256) {
+            const int g = i / a.e, c = i - g * a.e;
+            const size_t dst = (prow + (size_t)g * a.page) * a.e + c;
+            if (KVT == KV_F32) ((float*)a.vpool)[dst] = vv[i];
+            else ((uint16_t*)a.vpool)[dst] = f32_to_bf16(vv[i]);
+        }
+    }
+}
+void launch_lay_qk_prep(float* proj, int ldp, int q_off, int k_off, int v_off, int H, int G, int d, int e, const float* qn, const float* kn,
+                        float eps, int dims, bool half, const float* freq, float mag, void* kpool, void* vpool, int kvt, const int32_t* bt,
+                        const LaySegDev* segs, const int32_t* rowseg, int T, int page, hipStream_t s) {
+    if (T <= 0) return;
+    LQkPrepArgs a{proj, ldp, q_off, k_off, v_off, H, G, d, e, qn, kn, eps, freq ? dims : 0, half ? 1 : 0, freq, mag, kpool, vpool, bt, segs, rowseg, page};
+    if (kvt == KV_F32) hipLaunchKernelGGL(lay_qk_prep_kernel<KV_F32>, dim3((unsigned)T), dim3(256), 0, s, a);
+    else hipLaunchKernelGGL(lay_qk_prep_kernel<KV_BF16>, dim3((unsigned)T), dim3(256), 0, s, a);
 }
 
 // A block = 16 query rows of one sequence and one key head: row qi = (position in the portion) * nrep + (query head in the
@@ -1646,18 +1734,20 @@ void launch_lay_lightning(const LLightArgs& a, hipStream_t s) {
 // constant 1 as one more value column (so that the state's last column is n) this is the gated linear attention above; what is
 // left are the gates with their running maximum (here) and the division, head norm and output gate (lay_memory_out).
 // ------------------------------------------------------------------------------------------------------------------
-// One wave per (sequence, head).  x -> max(x + lf, li) composes: after (a1, b1) then (a2, b2) it is x -> max(x + a1 + a2, max(b1 + a2, b2)),
-// so the running maximum of 64 tokens comes from a shuffle scan over the lanes; the portion's last m goes back to the state.
-__global__ __launch_bounds__(64) void lay_memory_gates_kernel(const float* __restrict__ proj, int ldp, int i_off, int f_off, float cap,
-                                                              float* __restrict__ ldec, float* __restrict__ kmul, float* __restrict__ mrun,
-                                                              float* __restrict__ state_pool, size_t slot_stride, size_t m_off,
-                                                              const LaySegDev* __restrict__ segs, int H) {
+// One block per (sequence, head), 256 tokens a round.  x -> max(x + lf, li) composes: after (a1, b1) then (a2, b2) it is
+// x -> max(x + a1 + a2, max(b1 + a2, b2)), so the running maximum comes from a shuffle scan over each wave's 64 tokens and a
+// second step over the four waves' totals; the portion's last m goes back to the state.
+__global__ __launch_bounds__(256) void lay_memory_gates_kernel(const float* __restrict__ proj, int ldp, int i_off, int f_off, float cap,
+                                                               float* __restrict__ ldec, float* __restrict__ kmul, float* __restrict__ mrun,
+                                                               float* __restrict__ state_pool, size_t slot_stride, size_t m_off,
+                                                               const LaySegDev* __restrict__ segs, int H) {
+    __shared__ float wa[4], wb[4], carry;
     const LaySegDev sg = segs[blockIdx.x];
-    const int head = blockIdx.y, lane = threadIdx.x;
+    const int head = blockIdx.y, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     float* mp = state_pool + (size_t)sg.slot * slot_stride + m_off + head;
     float m = *mp;
-    for (int t0 = 0; t0 < sg.n; t0 += 64) {
-        const int t = t0 + lane;
+    for (int t0 = 0; t0 < sg.n; t0 += 256) {
+        const int t = t0 + tid;
         const bool ok = t < sg.n;
         float li = -INFINITY, lf = 0.f;            // past the portion: the identity x -> x
         if (ok) {
@@ -1671,23 +1761,29 @@ __global__ __launch_bounds__(64) void lay_memory_gates_kernel(const float* __res
             const float pa = __shfl_up(A, off), pb = __shfl_up(B, off);
             if (lane >= off) { B = fmaxf(pb + A, B); A = pa + A; }
         }
-        const float mt = fmaxf(m + A, B);
+        if (lane == 63) { wa[wave] = A; wb[wave] = B; }
+        __syncthreads();
+        float mw = m;                              // the running maximum in front of this wave's tokens
+        for (int w = 0; w < wave; ++w) mw = fmaxf(mw + wa[w], wb[w]);
+        const float mt = fmaxf(mw + A, B);
         float mprev = __shfl_up(mt, 1);
-        if (lane == 0) mprev = m;
+        if (lane == 0) mprev = mw;
         if (ok) {
             const size_t o = (size_t)(sg.row0 + t) * H + head;
             ldec[o] = lf + mprev - mt;
             kmul[o] = expf(li - mt);
             mrun[o] = mt;
         }
-        m = __shfl(mt, min(63, sg.n - t0 - 1));
+        if (tid == 255) carry = mt;                // tokens past the portion pass the last valid m through
+        __syncthreads();
+        m = carry;
     }
-    if (lane == 0) *mp = m;
+    if (tid == 0) *mp = m;
 }
 void launch_lay_memory_gates(const float* proj, int ldp, int i_off, int f_off, float cap, float* ldec, float* kmul, float* mrun,
                              float* state_pool, size_t slot_stride, size_t m_off, const LaySegDev* segs, int nseg, int H, hipStream_t s) {
     if (nseg <= 0 || H <= 0) return;
-    hipLaunchKernelGGL(lay_memory_gates_kernel, dim3((unsigned)nseg, (unsigned)H), dim3(64), 0, s, proj, ldp, i_off, f_off, cap, ldec, kmul, mrun,
+    hipLaunchKernelGGL(lay_memory_gates_kernel, dim3((unsigned)nseg, (unsigned)H), dim3(256), 0, s, proj, ldp, i_off, f_off, cap, ldec, kmul, mrun,
                        state_pool, slot_stride, m_off, segs, H);
 }
 // one wave per (row, head)
@@ -1719,7 +1815,7 @@ void launch_lay_memory_out(const float* o, const float* mrun, const float* gate,
 __global__ __launch_bounds__(256) void lay_router_kernel(const float* __restrict__ h, const uint16_t* __restrict__ wr, int32_t* __restrict__ sel,
                                                          float* __restrict__ wsel, int W, int E, int top, RouterSpec rs,
                                                          const float* __restrict__ correction, int slots) {
-    extern __shared__ float zs[];          // [E] logits, then choice scores; [E] scores
+    extern __shared__ float zs[];          // [E] logits, then choice scores; [E] scores; [groups]; [top]
     float* sc = zs + E;
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float* hr = h + (size_t)t * W;
@@ -1730,54 +1826,85 @@ __global__ __launch_bounds__(256) void lay_router_kernel(const float* __restrict
         if (lane == 0) zs[ex] = s;
     }
     __syncthreads();
-    if (threadIdx.x == 0) {
-        // scores; the choice goes by score + correction (plain sigmoid scores: by the logits themselves, the same order)
-        if (rs.softmax) {
-            float mx = -INFINITY, sum = 0.f;
-            for (int ex = 0; ex < E; ++ex) mx = fmaxf(mx, zs[ex]);
-            for (int ex = 0; ex < E; ++ex) { sc[ex] = expf(zs[ex] - mx); sum += sc[ex]; }
-            for (int ex = 0; ex < E; ++ex) sc[ex] /= sum;
-        } else
-            for (int ex = 0; ex < E; ++ex) sc[ex] = 1.f / (1.f + expf(-zs[ex]));
-        if (rs.softmax || correction)
-            for (int ex = 0; ex < E; ++ex) zs[ex] = sc[ex] + (correction ? correction[ex] : 0.f);
-        if (rs.groups > 1) {               // keep the best groups: every pass removes the worst remaining one
-            const int per = E / rs.groups;
-            for (int drop = 0; drop < rs.groups - rs.keep_groups; ++drop) {
-                int worst = -1; float wv = 0.f;
-                for (int g = rs.groups - 1; g >= 0; --g) {     // among equals the later group goes first
-                    float best = -INFINITY; bool live = false;
-                    for (int j = 0; j < per; ++j) { const float c = zs[g * per + j]; if (c != -INFINITY) live = true; best = fmaxf(best, c); }
-                    if (!live) continue;
-                    if (worst < 0 || best < wv) { worst = g; wv = best; }
-                }
-                if (worst < 0) break;
-                for (int j = 0; j < per; ++j) zs[worst * per + j] = -INFINITY;
-            }
+    if (wave != 0) return;
+    // wave 0: lane l owns outputs l, l + 64, ...; maxima, sums and the arg-max (lowest index among equals) are wave reductions
+    auto arg_best = [&](bool want_max, int lo, int hi, float& bv) {      // over the live (not -inf) entries of zs[lo, hi)
+        float v = 0.f; int at = 0x7fffffff;
+        for (int ex = lo + lane; ex < hi; ex += 64) {
+            const float z = zs[ex];
+            if (z == -INFINITY) continue;
+            if (at == 0x7fffffff || (want_max ? z > v : z < v)) { v = z; at = ex; }
         }
-        float wsum = 0.f;
-        for (int k = 0; k < top; ++k) {
-            int best = -1; float bz = 0.f;
-            for (int ex = 0; ex < E; ++ex) {
-                const float z = zs[ex];
-                if (z == -INFINITY) continue;
-                if (best < 0 || z > bz) { best = ex; bz = z; }
+        for (int off = 32; off > 0; off >>= 1) {
+            const float ov = __shfl_xor(v, off); const int oa = __shfl_xor(at, off);
+            if (oa != 0x7fffffff && (at == 0x7fffffff || (want_max ? ov > v : ov < v) || (ov == v && oa < at))) { v = ov; at = oa; }
+        }
+        bv = v;
+        return at;
+    };
+    // scores; the choice goes by score + correction (plain sigmoid scores: by the logits themselves, the same order)
+    if (rs.softmax) {
+        float mx = -INFINITY;
+        for (int ex = lane; ex < E; ex += 64) mx = fmaxf(mx, zs[ex]);
+        mx = wave_max(mx);
+        float sum = 0.f;
+        for (int ex = lane; ex < E; ex += 64) { const float p = expf(zs[ex] - mx); sc[ex] = p; sum += p; }
+        sum = wave_sum(sum);
+        for (int ex = lane; ex < E; ex += 64) sc[ex] /= sum;
+    } else
+        for (int ex = lane; ex < E; ex += 64) sc[ex] = 1.f / (1.f + expf(-zs[ex]));
+    if (rs.softmax || correction)
+        for (int ex = lane; ex < E; ex += 64) zs[ex] = sc[ex] + (correction ? correction[ex] : 0.f);
+    __builtin_amdgcn_wave_barrier();
+    if (rs.groups > 1) {                   // keep the best groups: every pass removes the worst remaining one
+        const int per = E / rs.groups;
+        float* gb = sc + E;                // [groups] a group's largest choice score (-inf: removed)
+        for (int g = lane; g < rs.groups; g += 64) {
+            float best = -INFINITY;
+            for (int j = 0; j < per; ++j) best = fmaxf(best, zs[g * per + j]);
+            gb[g] = best;
+        }
+        for (int drop = 0; drop < rs.groups - rs.keep_groups; ++drop) {
+            // the worst live group, among equals the last one
+            float v = 0.f; int at = -1;
+            for (int g = lane; g < rs.groups; g += 64) {
+                const float b = gb[g];
+                if (b == -INFINITY) continue;
+                if (at < 0 || b <= v) { v = b; at = g; }
             }
-            if (best < 0) { best = 0; }
+            for (int off = 32; off > 0; off >>= 1) {
+                const float ov = __shfl_xor(v, off); const int oa = __shfl_xor(at, off);
+                if (oa >= 0 && (at < 0 || ov < v || (ov == v && oa > at))) { v = ov; at = oa; }
+            }
+            if (at < 0) break;
+            if (lane == 0) gb[at] = -INFINITY;
+            for (int j = lane; j < per; j += 64) zs[at * per + j] = -INFINITY;
+            __builtin_amdgcn_wave_barrier();      // LDS accesses of one wave complete in order; this keeps the compiler from moving them
+        }
+    }
+    float* wl = sc + E + rs.groups;        // [top] the chosen scores
+    float wsum = 0.f;
+    for (int k = 0; k < top; ++k) {
+        float bz;
+        int best = arg_best(true, 0, E, bz);
+        if (best == 0x7fffffff) best = 0;
+        const float w = sc[best];
+        wsum += w;
+        if (lane == 0) {
             sel[(size_t)t * top + k] = best;
-            wsel[(size_t)t * slots + k] = sc[best];
-            wsum += sc[best];
+            wl[k] = w;
             zs[best] = -INFINITY;
         }
-        if (rs.normalise) for (int k = 0; k < top; ++k) wsel[(size_t)t * slots + k] /= wsum + 1e-20f;
-        for (int k = top; k < slots; ++k) wsel[(size_t)t * slots + k] = 1.f;
+        __builtin_amdgcn_wave_barrier();
     }
+    for (int k = lane; k < top; k += 64) wsel[(size_t)t * slots + k] = rs.normalise ? wl[k] / (wsum + 1e-20f) : wl[k];
+    for (int k = top + lane; k < slots; k += 64) wsel[(size_t)t * slots + k] = 1.f;
 }
 void launch_lay_router(const float* h, const uint16_t* wr, int32_t* sel, float* wsel, int T, int W, int E, int top, hipStream_t s,
                        const RouterSpec* rs, const float* correction, int slots) {
     if (T <= 0) return;
     const RouterSpec r = rs ? *rs : RouterSpec();
-    hipLaunchKernelGGL(lay_router_kernel, dim3((unsigned)T), dim3(256), (size_t)2 * E * sizeof(float), s, h, wr, sel, wsel, W, E, top, r,
+    hipLaunchKernelGGL(lay_router_kernel, dim3((unsigned)T), dim3(256), (size_t)(2 * E + r.groups + top) * sizeof(float), s, h, wr, sel, wsel, W, E, top, r,
                        r.correction ? correction : nullptr, slots > top ? slots : top);
 }
 

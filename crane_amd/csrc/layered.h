@@ -207,8 +207,15 @@ void launch_lay_k_append(const float* proj, int ldp, int k_off, void* kpool, int
                          const int32_t* rowseg, int T, int G, int d, int page, hipStream_t s);
 // mean key (and value) rows of the position blocks that the pass completes: block b of `pool` positions lives in the page of its
 // last position, row b - (first block that ends in that page).  Reads the cached rows, so it follows lay_k_append.
-void launch_lay_pool_append(const void* kpool, void* pk_pool, int kvt, const int32_t* bt, const LaySegDev* segs, const int32_t* rowseg, int T,
-                            int G, int d, int page, int pool, int pool_rows, hipStream_t s);
+// Keys [..][d] and -- vpool given -- values [..][e] in one launch.
+void launch_lay_pool_append(const void* kpool, void* pk_pool, int d, const void* vpool, void* pv_pool, int e, int kvt, const int32_t* bt,
+                            const LaySegDev* segs, const int32_t* rowseg, int T, int G, int page, int pool, int pool_rows, hipStream_t s);
+// queries and keys of a pass on their way into attention, one launch: RMS norm over all query heads at once and over all key heads
+// at once (qn / kn: weights [H d] / [G d]; null: no norm), rotation by position (freq null: none), q back in place, keys -- and
+// values, vpool given -- into the pages
+void launch_lay_qk_prep(float* proj, int ldp, int q_off, int k_off, int v_off, int H, int G, int d, int e, const float* qn, const float* kn,
+                        float eps, int dims, bool half, const float* freq, float mag, void* kpool, void* vpool, int kvt, const int32_t* bt,
+                        const LaySegDev* segs, const int32_t* rowseg, int T, int page, hipStream_t s);
 inline int lay_pool_rows(int page, long long pool) { return pool >= page ? 1 : (int)((page + pool - 1) / pool); }
 void launch_lay_attn(const LAttnArgs& a, int kvt, hipStream_t s);    // kvt: KV_BF16 | KV_F32
 bool lay_attn_fits(int d, int e, bool own_v);                         // sizes the kernel can hold in LDS and registers

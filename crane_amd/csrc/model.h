@@ -427,6 +427,7 @@ int prefill_lo_mask = 0;              // EXPERIMENT (cm_debug_set "prefill_lo_ma
     void layered_set_capture(bool on);                    // cm_debug_set("lay_capture")
     void layered_set_shared_gemm(bool on);                // cm_debug_set("lay_shared_gemm")
     void layered_set_attn_mfma(bool on);                  // cm_debug_set("lay_attn_mfma")
+    void layered_set_fused_prep(bool on);                 // cm_debug_set("lay_fused_prep")
     size_t layered_capture(float* out, size_t n) const;   // cm_debug_read("lay_layers"): [pass][layer][row][width]; returns the count
 
     // ---- construction ----

@@ -49,6 +49,7 @@ struct Layered {
     // families' prompt passes use (kernels_prefill.hip / kernels_gemm256.hip), plain bf16 activations; cm_debug_set("lay_shared_gemm", 0): never
     bool shared_gemm = true;
     bool attn_mfma = true;             // bfloat16 format, prompt passes: the matrix-core attention (cm_debug_set("lay_attn_mfma", 0): never)
+    bool fused_prep = true;            // query / key norm + rotation + cache append in one launch (cm_debug_set("lay_fused_prep", 0): single operations)
     uint16_t* Abf = nullptr;           // [cap rounded up to 256][widest K] bf16 A operand
     float *G1 = nullptr, *G2 = nullptr;   // [cap][widest dense ff] the two products of a gated feed-forward
     float* U = nullptr;                // lightning attention, chunk-parallel form: [chunks of a pass][widest H d e] f32
@@ -949,6 +950,10 @@ void Model::layered_set_attn_mfma(bool on) {
     if (!lay) throw CmError(CM_ERR_UNSUPPORTED, "not a layer-list decoder");
     lay->attn_mfma = on;
 }
+void Model::layered_set_fused_prep(bool on) {
+    if (!lay) throw CmError(CM_ERR_UNSUPPORTED, "not a layer-list decoder");
+    lay->fused_prep = on;
+}
 void Model::layered_set_capture(bool on) {
     if (!lay) throw CmError(CM_ERR_UNSUPPORTED, "not a layer-list decoder");
     lay->capture = on;
@@ -1265,24 +1270,27 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                     const LayeredLayerW& sw = w.side[k];
                     const int H = sd.heads, G = sd.kv_heads, d = sd.dim, e = sd.vdim;
                     if (sd.mixer == LMIX_ATTN) {
-                        if (sd.qk_norm) {
-                            launch_lay_rms_cols(L.P, w.in_rows, sw.q_off, H * d, sw.q_norm, L.P + sw.q_off, w.in_rows, T, cfg.eps, s);
-                            launch_lay_rms_cols(L.P, w.in_rows, sw.k_off, G * d, sw.k_norm, L.P + sw.k_off, w.in_rows, T, cfg.eps, s);
+                        if (L.fused_prep) {
+                            launch_lay_qk_prep(L.P, w.in_rows, sw.q_off, sw.k_off, sw.v_off, H, G, d, e, sd.qk_norm ? sw.q_norm : nullptr,
+                                               sd.qk_norm ? sw.k_norm : nullptr, cfg.eps, sd.rot.dims, sd.rot.half, sd.rot.dims > 0 ? sw.rot_freq : nullptr,
+                                               sw.rot_mag, kv_pool + sw.k_pool_off, kv_pool + sw.v_pool_off, kv_mode, d_bt, d_segs, d_rowseg, T, page, s);
+                        } else {               // the same from the single operations
+                            if (sd.qk_norm) {
+                                launch_lay_rms_cols(L.P, w.in_rows, sw.q_off, H * d, sw.q_norm, L.P + sw.q_off, w.in_rows, T, cfg.eps, s);
+                                launch_lay_rms_cols(L.P, w.in_rows, sw.k_off, G * d, sw.k_norm, L.P + sw.k_off, w.in_rows, T, cfg.eps, s);
+                            }
+                            if (sd.rot.dims > 0) {
+                                launch_lay_rope(L.P + sw.q_off, w.in_rows, d, L.P + sw.q_off, w.in_rows, d, H, d, sd.rot.dims, sw.rot_freq, sw.rot_mag,
+                                                d_segs, d_rowseg, T, s, sd.rot.half);
+                                launch_lay_rope(L.P + sw.k_off, w.in_rows, d, L.P + sw.k_off, w.in_rows, d, G, d, sd.rot.dims, sw.rot_freq, sw.rot_mag,
+                                                d_segs, d_rowseg, T, s, sd.rot.half);
+                            }
+                            launch_lay_k_append(L.P, w.in_rows, sw.k_off, kv_pool + sw.k_pool_off, kv_mode, d_bt, d_segs, d_rowseg, T, G, d, page, s);
+                            launch_lay_k_append(L.P, w.in_rows, sw.v_off, kv_pool + sw.v_pool_off, kv_mode, d_bt, d_segs, d_rowseg, T, G, e, page, s);
                         }
-                        if (sd.rot.dims > 0) {
-                            launch_lay_rope(L.P + sw.q_off, w.in_rows, d, L.P + sw.q_off, w.in_rows, d, H, d, sd.rot.dims, sw.rot_freq, sw.rot_mag,
-                                            d_segs, d_rowseg, T, s, sd.rot.half);
-                            launch_lay_rope(L.P + sw.k_off, w.in_rows, d, L.P + sw.k_off, w.in_rows, d, G, d, sd.rot.dims, sw.rot_freq, sw.rot_mag,
-                                            d_segs, d_rowseg, T, s, sd.rot.half);
-                        }
-                        launch_lay_k_append(L.P, w.in_rows, sw.k_off, kv_pool + sw.k_pool_off, kv_mode, d_bt, d_segs, d_rowseg, T, G, d, page, s);
-                        launch_lay_k_append(L.P, w.in_rows, sw.v_off, kv_pool + sw.v_pool_off, kv_mode, d_bt, d_segs, d_rowseg, T, G, e, page, s);
-                        if (sd.pool > 0) {
-                            launch_lay_pool_append(kv_pool + sw.k_pool_off, kv_pool + sw.pk_pool_off, kv_mode, d_bt, d_segs, d_rowseg, T, G, d, page,
-                                                   (int)sd.pool, sw.pool_rows, s);
-                            launch_lay_pool_append(kv_pool + sw.v_pool_off, kv_pool + sw.pv_pool_off, kv_mode, d_bt, d_segs, d_rowseg, T, G, e, page,
-                                                   (int)sd.pool, sw.pool_rows, s);
-                        }
+                        if (sd.pool > 0)
+                            launch_lay_pool_append(kv_pool + sw.k_pool_off, kv_pool + sw.pk_pool_off, d, kv_pool + sw.v_pool_off, kv_pool + sw.pv_pool_off, e,
+                                                   kv_mode, d_bt, d_segs, d_rowseg, T, G, page, (int)sd.pool, sw.pool_rows, s);
                         run_attention(sd, sw, L.P, w.in_rows, sw.q_off, 0, d, e, L.O + sw.o_col, ocols, sd.side_scale);
                     } else if (sd.mixer == LMIX_MEMORY) {
                         launch_lay_memory_gates(L.P, w.in_rows, sw.i_off, sw.f_off, sd.gate_cap, L.LD, L.KM, L.MR, state_pool, state_slot_elems,

@@ -462,6 +462,22 @@ def test_matrix_core_attention_of_prompt_passes_against_the_plain_kernel(tmp_pat
         m.close()
 
 
+def test_single_operations_in_place_of_the_fused_query_and_key_preparation(tmp_path):
+    cfg = U.small_config()
+    P = U.random_weights(cfg, 18)
+    toks = U.tokens(90, cfg["vocab"], 18)
+    want = O.forward(cfg, P, toks)
+    m = _load(tmp_path, cfg, P)
+    try:
+        m.debug_set("lay_fused_prep", 0)
+        a = m.seq_alloc()
+        got = [m.step_batch([(a, toks[:60], _all(60))])[0]]
+        got += [m.step_batch([(a, [t], [0])])[0] for t in toks[60:]]
+        assert _err(np.concatenate(got), want) < TOL_F32
+    finally:
+        m.close()
+
+
 def _drawn_config(seed):
     """A model of this design with sizes, windows, block lengths and constants drawn from the seed."""
     rs = np.random.RandomState(100 + seed)
