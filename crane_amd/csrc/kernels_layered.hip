@@ -238,34 +238,60 @@ void launch_lay_rms_gate(const float* o, const float* gate, int ldg, const float
     hipLaunchKernelGGL(lay_rms_gate_kernel, dim3((unsigned)T), dim3(256), 0, s, o, gate, ldg, w, out, N, eps);
 }
 
+// the combined expert rows of token r at channel c: sum_k wsel[r top + k] * row_k, row_k = ys[(r top + k) W + c] or -- choices k < sel_top
+// whose expert index is an identity expert (>= n_real) -- the sublayer's input hin[r W + c]
+struct LCombine { const float* wsel; int top; const int32_t* sel; int sel_top, n_real; const float* hin; };
+__device__ __forceinline__ float lay_combined(const float* __restrict__ y, const LCombine& cb, int r, int c, int W) {
+    if (!cb.wsel) return y[(size_t)r * W + c];
+    float v = 0.f;
+    for (int k = 0; k < cb.top; ++k) {
+        const bool ident = cb.sel && k < cb.sel_top && cb.sel[(size_t)r * cb.sel_top + k] >= cb.n_real;
+        v += cb.wsel[(size_t)r * cb.top + k] * (ident ? cb.hin[(size_t)r * W + c] : y[((size_t)r * cb.top + k) * W + c]);
+    }
+    return v;
+}
 __global__ __launch_bounds__(256) void lay_post_norm_kernel(float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ w,
-                                                            float mult, float eps, int W, const float* __restrict__ wsel, int top) {
+                                                            float mult, float eps, int W, LCombine cb) {
     __shared__ float red[4];
     const int r = blockIdx.x;
     float ss = 0.f;
-    for (int c = threadIdx.x; c < W; c += 256) {
-        float v;
-        if (wsel) {
-            v = 0.f;
-            for (int k = 0; k < top; ++k) v += wsel[(size_t)r * top + k] * y[((size_t)r * top + k) * W + c];
-        } else v = y[(size_t)r * W + c];
-        ss += v * v;
+    for (int c = threadIdx.x; c < W; c += 256) { const float v = lay_combined(y, cb, r, c, W); ss += v * v; }
+    ss = block_sum(ss, red);
+    const float rs = 1.f / sqrtf(ss / (float)W + eps);
+    for (int c = threadIdx.x; c < W; c += 256) x[(size_t)r * W + c] += mult * (lay_combined(y, cb, r, c, W) * rs * w[c]);
+}
+// rows of up to 256 EPT channels: the combined values are formed once and wait in registers for the root mean square
+template <int EPT>
+__global__ __launch_bounds__(256) void lay_post_norm_reg_kernel(float* __restrict__ x, const float* __restrict__ y, const float* __restrict__ w,
+                                                                float mult, float eps, int W, LCombine cb) {
+    __shared__ float red[4];
+    const int r = blockIdx.x;
+    float yv[EPT], xv[EPT], wv[EPT];
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+        const int c = threadIdx.x + 256 * e;
+        const bool ok = c < W;
+        yv[e] = ok ? lay_combined(y, cb, r, c, W) : 0.f;
+        xv[e] = ok ? x[(size_t)r * W + c] : 0.f;
+        wv[e] = ok ? w[c] : 0.f;
+        ss += yv[e] * yv[e];
     }
     ss = block_sum(ss, red);
     const float rs = 1.f / sqrtf(ss / (float)W + eps);
-    for (int c = threadIdx.x; c < W; c += 256) {
-        float v;
-        if (wsel) {
-            v = 0.f;
-            for (int k = 0; k < top; ++k) v += wsel[(size_t)r * top + k] * y[((size_t)r * top + k) * W + c];
-        } else v = y[(size_t)r * W + c];
-        x[(size_t)r * W + c] += mult * (v * rs * w[c]);
+#pragma unroll
+    for (int e = 0; e < EPT; ++e) {
+        const int c = threadIdx.x + 256 * e;
+        if (c < W) x[(size_t)r * W + c] = xv[e] + mult * (yv[e] * rs * wv[e]);
     }
 }
 void launch_lay_post_norm(float* x, const float* y, const float* w, float mult, float eps, int T, int W, const float* wsel, int top,
-                          hipStream_t s) {
+                          hipStream_t s, const int32_t* sel, int sel_top, int n_real, const float* hin) {
     if (T <= 0) return;
-    hipLaunchKernelGGL(lay_post_norm_kernel, dim3((unsigned)T), dim3(256), 0, s, x, y, w, mult, eps, W, wsel, top);
+    const LCombine cb{wsel, top, n_real >= 0 && hin ? sel : nullptr, sel_top, n_real, hin};
+    if (W <= 1024) hipLaunchKernelGGL(lay_post_norm_reg_kernel<4>, dim3((unsigned)T), dim3(256), 0, s, x, y, w, mult, eps, W, cb);
+    else if (W <= 4096) hipLaunchKernelGGL(lay_post_norm_reg_kernel<16>, dim3((unsigned)T), dim3(256), 0, s, x, y, w, mult, eps, W, cb);
+    else hipLaunchKernelGGL(lay_post_norm_kernel, dim3((unsigned)T), dim3(256), 0, s, x, y, w, mult, eps, W, cb);
 }
 
 // ------------------------------------------------------------------------------------------------------------------
@@ -841,6 +867,26 @@ __device__ __forceinline__ LaRow la_row(const LAttnArgs& a, const LaySegDev& sg,
     return r;
 }
 
+// the mean row of the block of `pool` positions that ends at pos: f32 sum in position order, one rounding into the cache's format
+template <int KVT>
+__device__ __forceinline__ void lay_block_mean(const void* __restrict__ src, void* __restrict__ dstp, int n, const int32_t* __restrict__ bt,
+                                               int bt_off, int pos, int G, int page, int pool, int pool_rows) {
+    const int b = (pos + 1) / pool - 1, lpg = pos / page;
+    const int idx = b - (int)(((long long)lpg * page) / pool);
+    const float inv = 1.f / (float)pool;
+    for (int i = threadIdx.x; i < G * n; i += 256) {
+        const int g = i / n, c = i - g * n;
+        float sum = 0.f;
+#pragma unroll 8
+        for (int j = b * pool; j <= pos; ++j) {
+            const size_t at = (((size_t)bt[bt_off + j / page] * G + g) * page + (size_t)(j % page)) * n + c;
+            sum += KVT == KV_F32 ? ((const float*)src)[at] : bf16_to_f32(((const uint16_t*)src)[at]);
+        }
+        const size_t dst = (((size_t)bt[bt_off + lpg] * G + g) * pool_rows + idx) * n + c;
+        if (KVT == KV_F32) ((float*)dstp)[dst] = sum * inv;
+        else ((uint16_t*)dstp)[dst] = f32_to_bf16(sum * inv);
+    }
+}
 // one block per row of the pass (blockIdx.y: keys / values); a row whose position closes a block of `pool` positions writes the block's
 // mean row (f32 sum in position order, then one rounding into the cache's format)
 template <int KVT>
@@ -852,24 +898,8 @@ __global__ __launch_bounds__(256) void lay_pool_append_kernel(const void* __rest
     const LaySegDev sg = segs[rowseg[r]];
     const int pos = sg.start_pos + (r - sg.row0);
     if ((pos + 1) % pool != 0) return;
-    const void* src = blockIdx.y ? vpool : kpool;
-    void* dstp = blockIdx.y ? pv_pool : pk_pool;
-    const int n = blockIdx.y ? e : d;
-    const int b = (pos + 1) / pool - 1, lpg = pos / page;
-    const int idx = b - (int)(((long long)lpg * page) / pool);
-    const float inv = 1.f / (float)pool;
-    for (int i = threadIdx.x; i < G * n; i += 256) {
-        const int g = i / n, c = i - g * n;
-        float sum = 0.f;
-#pragma unroll 8
-        for (int j = b * pool; j <= pos; ++j) {
-            const size_t at = (((size_t)bt[sg.bt_off + j / page] * G + g) * page + (size_t)(j % page)) * n + c;
-            sum += KVT == KV_F32 ? ((const float*)src)[at] : bf16_to_f32(((const uint16_t*)src)[at]);
-        }
-        const size_t dst = (((size_t)bt[sg.bt_off + lpg] * G + g) * pool_rows + idx) * n + c;
-        if (KVT == KV_F32) ((float*)dstp)[dst] = sum * inv;
-        else ((uint16_t*)dstp)[dst] = f32_to_bf16(sum * inv);
-    }
+    if (blockIdx.y) lay_block_mean<KVT>(vpool, pv_pool, e, bt, sg.bt_off, pos, G, page, pool, pool_rows);
+    else lay_block_mean<KVT>(kpool, pk_pool, d, bt, sg.bt_off, pos, G, page, pool, pool_rows);
 }
 void launch_lay_pool_append(const void* kpool, void* pk_pool, int d, const void* vpool, void* pv_pool, int e, int kvt, const int32_t* bt,
                             const LaySegDev* segs, const int32_t* rowseg, int T, int G, int page, int pool, int pool_rows, hipStream_t s) {
@@ -889,6 +919,9 @@ struct LQkPrepArgs {
     int dims, half; const float* freq; float mag;
     void *kpool, *vpool;
     const int32_t* bt; const LaySegDev* segs; const int32_t* rowseg; int page;
+    // pool > 0: every portion of the pass is ONE token, and a row that closes a block of `pool` positions also writes the block's mean
+    // rows (the other positions of the block were cached by earlier passes; its own by this block)
+    int pool, pool_rows; void *pk_pool, *pv_pool;
 };
 template <int KVT>
 __global__ __launch_bounds__(256) void lay_qk_prep_kernel(LQkPrepArgs a) {
@@ -950,12 +983,20 @@ __global__ __launch_bounds__(256) void lay_qk_prep_kernel(LQkPrepArgs a) {
             else ((uint16_t*)a.vpool)[dst] = f32_to_bf16(vv[i]);
         }
     }
+    if (a.pool > 0 && (pos + 1) % a.pool == 0) {
+        __threadfence_block();             // this block's own cached row is read back below
+        __syncthreads();
+        lay_block_mean<KVT>(a.kpool, a.pk_pool, a.d, a.bt, sg.bt_off, pos, a.G, a.page, a.pool, a.pool_rows);
+        if (a.vpool && a.pv_pool) lay_block_mean<KVT>(a.vpool, a.pv_pool, a.e, a.bt, sg.bt_off, pos, a.G, a.page, a.pool, a.pool_rows);
+    }
 }
 void launch_lay_qk_prep(float* proj, int ldp, int q_off, int k_off, int v_off, int H, int G, int d, int e, const float* qn, const float* kn,
                         float eps, int dims, bool half, const float* freq, float mag, void* kpool, void* vpool, int kvt, const int32_t* bt,
-                        const LaySegDev* segs, const int32_t* rowseg, int T, int page, hipStream_t s) {
+                        const LaySegDev* segs, const int32_t* rowseg, int T, int page, hipStream_t s, int pool, int pool_rows, void* pk_pool,
+                        void* pv_pool) {
     if (T <= 0) return;
-    LQkPrepArgs a{proj, ldp, q_off, k_off, v_off, H, G, d, e, qn, kn, eps, freq ? dims : 0, half ? 1 : 0, freq, mag, kpool, vpool, bt, segs, rowseg, page};
+    LQkPrepArgs a{proj, ldp, q_off, k_off, v_off, H, G, d, e, qn, kn, eps, freq ? dims : 0, half ? 1 : 0, freq, mag, kpool, vpool, bt, segs, rowseg, page,
+                  pk_pool ? pool : 0, pool_rows, pk_pool, pv_pool};
     if (kvt == KV_F32) hipLaunchKernelGGL(lay_qk_prep_kernel<KV_F32>, dim3((unsigned)T), dim3(256), 0, s, a);
     else hipLaunchKernelGGL(lay_qk_prep_kernel<KV_BF16>, dim3((unsigned)T), dim3(256), 0, s, a);
 }
@@ -1812,21 +1853,11 @@ void launch_lay_memory_out(const float* o, const float* mrun, const float* gate,
 // ------------------------------------------------------------------------------------------------------------------
 // mixture of experts: router + counting sort
 // ------------------------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void lay_router_kernel(const float* __restrict__ h, const uint16_t* __restrict__ wr, int32_t* __restrict__ sel,
-                                                         float* __restrict__ wsel, int W, int E, int top, RouterSpec rs,
-                                                         const float* __restrict__ correction, int slots) {
-    extern __shared__ float zs[];          // [E] logits, then choice scores; [E] scores; [groups]; [top]
+// One wave turns the E logits of token t in zs into choices and weights.  zs: [E] logits, then choice scores; sc = zs + E: [E] scores,
+// [groups], [top].
+__device__ __forceinline__ void lay_router_choose(float* zs, int t, int lane, int32_t* __restrict__ sel, float* __restrict__ wsel, int E, int top,
+                                                  const RouterSpec& rs, const float* __restrict__ correction, int slots) {
     float* sc = zs + E;
-    const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const float* hr = h + (size_t)t * W;
-    for (int ex = wave; ex < E; ex += 4) {
-        float s = 0.f;
-        for (int i = lane; i < W; i += 64) s = fmaf(hr[i], bf16_to_f32(wr[(size_t)ex * W + i]), s);
-        s = wave_sum(s);
-        if (lane == 0) zs[ex] = s;
-    }
-    __syncthreads();
-    if (wave != 0) return;
     // wave 0: lane l owns outputs l, l + 64, ...; maxima, sums and the arg-max (lowest index among equals) are wave reductions
     auto arg_best = [&](bool want_max, int lo, int hi, float& bv) {      // over the live (not -inf) entries of zs[lo, hi)
         float v = 0.f; int at = 0x7fffffff;
@@ -1900,10 +1931,48 @@ __global__ __launch_bounds__(256) void lay_router_kernel(const float* __restrict
     for (int k = lane; k < top; k += 64) wsel[(size_t)t * slots + k] = rs.normalise ? wl[k] / (wsum + 1e-20f) : wl[k];
     for (int k = top + lane; k < slots; k += 64) wsel[(size_t)t * slots + k] = 1.f;
 }
+// logits and choice in one launch, one block per token
+__global__ __launch_bounds__(256) void lay_router_kernel(const float* __restrict__ h, const uint16_t* __restrict__ wr, int32_t* __restrict__ sel,
+                                                         float* __restrict__ wsel, int W, int E, int top, RouterSpec rs,
+                                                         const float* __restrict__ correction, int slots) {
+    extern __shared__ float zs[];
+    const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const float* hr = h + (size_t)t * W;
+    for (int ex = wave; ex < E; ex += 4) {
+        float s = 0.f;
+        for (int i = lane; i < W; i += 64) s = fmaf(hr[i], bf16_to_f32(wr[(size_t)ex * W + i]), s);
+        s = wave_sum(s);
+        if (lane == 0) zs[ex] = s;
+    }
+    __syncthreads();
+    if (wave == 0) lay_router_choose(zs, t, lane, sel, wsel, E, top, rs, correction, slots);
+}
+// the choice from logits z [T][E] that a projection left: one wave per token
+__global__ __launch_bounds__(256) void lay_router_choose_kernel(const float* __restrict__ z, int32_t* __restrict__ sel, float* __restrict__ wsel, int T,
+                                                                int E, int top, RouterSpec rs, const float* __restrict__ correction, int slots,
+                                                                int per_wave) {
+    extern __shared__ float zs[];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int t = blockIdx.x * 4 + wave;
+    if (t >= T) return;
+    float* mine = zs + (size_t)wave * per_wave;
+    for (int ex = lane; ex < E; ex += 64) mine[ex] = z[(size_t)t * E + ex];
+    __builtin_amdgcn_wave_barrier();
+    lay_router_choose(mine, t, lane, sel, wsel, E, top, rs, correction, slots);
+}
 void launch_lay_router(const float* h, const uint16_t* wr, int32_t* sel, float* wsel, int T, int W, int E, int top, hipStream_t s,
-                       const RouterSpec* rs, const float* correction, int slots) {
+                       const RouterSpec* rs, const float* correction, int slots, float* zbuf) {
     if (T <= 0) return;
     const RouterSpec r = rs ? *rs : RouterSpec();
+    if (zbuf && T <= LV_MAXM) {            // decode steps: logits by the streaming row kernel in f32 (every wave busy), then the choice
+        LGemmArgs g;
+        g.A = h; g.lda = W; g.W = wr; g.C = zbuf; g.ldc = E; g.M = T; g.N = E; g.K = W;
+        launch_lgemm(g, false, 1, s);
+        const int per_wave = 2 * E + r.groups + top;
+        hipLaunchKernelGGL(lay_router_choose_kernel, dim3((unsigned)((T + 3) / 4)), dim3(256), (size_t)4 * per_wave * sizeof(float), s, zbuf, sel, wsel,
+                           T, E, top, r, r.correction ? correction : nullptr, slots > top ? slots : top, per_wave);
+        return;
+    }
     hipLaunchKernelGGL(lay_router_kernel, dim3((unsigned)T), dim3(256), (size_t)(2 * E + r.groups + top) * sizeof(float), s, h, wr, sel, wsel, W, E, top, r,
                        r.correction ? correction : nullptr, slots > top ? slots : top);
 }
@@ -1925,17 +1994,6 @@ __global__ __launch_bounds__(1024) void lay_moe_plan_kernel(const int32_t* __res
 }
 void launch_lay_moe_plan(const int32_t* sel, int32_t* off, int32_t* srt, int n, int E, hipStream_t s, int top, int slots) {
     hipLaunchKernelGGL(lay_moe_plan_kernel, dim3(1), dim3(1024), (size_t)E * sizeof(int), s, sel, off, srt, n, E, top, slots);
-}
-__global__ __launch_bounds__(256) void lay_moe_identity_kernel(const int32_t* __restrict__ sel, const float* __restrict__ h, float* __restrict__ ys,
-                                                               int W, int top, int slots, int n_real) {
-    const int p = blockIdx.x;
-    if (sel[p] < n_real) return;
-    const int t = p / top, k = p - t * top;
-    for (int c = threadIdx.x; c < W; c += 256) ys[((size_t)t * slots + k) * W + c] = h[(size_t)t * W + c];
-}
-void launch_lay_moe_identity(const int32_t* sel, const float* h, float* ys, int T, int W, int top, int slots, int n_real, hipStream_t s) {
-    if (T <= 0 || top <= 0) return;
-    hipLaunchKernelGGL(lay_moe_identity_kernel, dim3((unsigned)(T * top)), dim3(256), 0, s, sel, h, ys, W, top, slots, n_real);
 }
 
 // arg-max of every row, lowest index among equals

@@ -179,9 +179,10 @@ void launch_lay_norm_canon_decode(const float* x, const float* nw, float eps, fl
 void launch_lay_post_norm_canon_decode(float* x, const float* y, const float* pw, float mult, const float* wsel, int top, const float* nw,
                                        float eps, float* out, const float* cw, float* conv_pool, size_t slot_stride, size_t off,
                                        const LaySegDev* segs, int T, int W, int taps, hipStream_t s);
-// x += mult * RMSNorm(y) * w;  sel != null: y[r] = sum_k wsel[r top + k] * ys[r top + k] (mixture-of-experts combine)
+// x += mult * RMSNorm(y) * w;  wsel != null: y[r] = sum_k wsel[r top + k] * ys[r top + k] (mixture-of-experts combine); hin given: the
+// rows of choices k < sel_top with sel[r sel_top + k] >= n_real are hin[r] (identity experts)
 void launch_lay_post_norm(float* x, const float* y, const float* w, float mult, float eps, int T, int W, const float* wsel, int top,
-                          hipStream_t s);
+                          hipStream_t s, const int32_t* sel = nullptr, int sel_top = 0, int n_real = -1, const float* hin = nullptr);
 
 struct LAttnArgs {
     const float* proj; int ldp, q_off, g_off;        // activated projection rows: q | k | gate
@@ -212,10 +213,12 @@ void launch_lay_pool_append(const void* kpool, void* pk_pool, int d, const void*
                             const LaySegDev* segs, const int32_t* rowseg, int T, int G, int page, int pool, int pool_rows, hipStream_t s);
 // queries and keys of a pass on their way into attention, one launch: RMS norm over all query heads at once and over all key heads
 // at once (qn / kn: weights [H d] / [G d]; null: no norm), rotation by position (freq null: none), q back in place, keys -- and
-// values, vpool given -- into the pages
+// values, vpool given -- into the pages.  pk_pool given (only when every portion of the pass is one token): the mean rows of a block that
+// the row closes, as lay_pool_append
 void launch_lay_qk_prep(float* proj, int ldp, int q_off, int k_off, int v_off, int H, int G, int d, int e, const float* qn, const float* kn,
                         float eps, int dims, bool half, const float* freq, float mag, void* kpool, void* vpool, int kvt, const int32_t* bt,
-                        const LaySegDev* segs, const int32_t* rowseg, int T, int page, hipStream_t s);
+                        const LaySegDev* segs, const int32_t* rowseg, int T, int page, hipStream_t s, int pool = 0, int pool_rows = 0,
+                        void* pk_pool = nullptr, void* pv_pool = nullptr);
 inline int lay_pool_rows(int page, long long pool) { return pool >= page ? 1 : (int)((page + pool - 1) / pool); }
 void launch_lay_attn(const LAttnArgs& a, int kvt, hipStream_t s);    // kvt: KV_BF16 | KV_F32
 bool lay_attn_fits(int d, int e, bool own_v);                         // sizes the kernel can hold in LDS and registers
@@ -256,12 +259,12 @@ void launch_lay_rms_gate(const float* o, const float* gate, int ldg, const float
 // router: z = h . Wr^T in f32 over E outputs, scores by rs (sigmoid of each / softmax over all), the `top` largest choice scores
 // (score + correction, inside the best groups; lowest index first among equals) -> sel [T top], wsel [T slots] = their scores
 // (normalised when asked); slots > top: the remaining weights are 1 (rows that every token uses, e.g. a shared expert)
+// zbuf [T][E] given and few rows (decode steps): the logits come from the streaming row kernel (f32 products of the unrounded rows),
+// then one wave per token chooses; otherwise one block per token does both
 void launch_lay_router(const float* h, const uint16_t* wr, int32_t* sel, float* wsel, int T, int W, int E, int top, hipStream_t s,
-                       const RouterSpec* rs = nullptr, const float* correction = nullptr, int slots = 0);
+                       const RouterSpec* rs = nullptr, const float* correction = nullptr, int slots = 0, float* zbuf = nullptr);
 // counting sort of the T top (token, choice) pairs by expert: off [E + 1], srt [T top] = token * slots + choice
 void launch_lay_moe_plan(const int32_t* sel, int32_t* off, int32_t* srt, int n, int E, hipStream_t s, int top = 1, int slots = 1);
-// rows of the identity experts: ys[token * slots + choice] = h[token] where sel >= n_real
-void launch_lay_moe_identity(const int32_t* sel, const float* h, float* ys, int T, int W, int top, int slots, int n_real, hipStream_t s);
 
 // matrix memory, gates: per (sequence, head) over the portion's tokens, from the pre-activations zi, zf at proj[t ldp + i_off / f_off + head]
 //   li = cap tanh(zi / cap), lf = ln sigmoid(cap tanh(zf / cap)), m' = max(lf + m, li)  (m: per-sequence state at mstate, [H])

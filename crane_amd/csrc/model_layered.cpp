@@ -29,6 +29,7 @@ struct Layered {
     bool post_only = false;
     float embed_scale = 1.f, logit_scale = 1.f;
     int max_mh = 0, max_sff = 0, max_slots = 1;   // matrix-memory heads, shared expert size, rows per token of an expert combine
+    float* Z = nullptr;                // router logits [cap][most outputs]
     float *KM = nullptr, *MR = nullptr, *HS = nullptr;   // matrix memory: key factor and running maximum per token and head; shared expert's inner rows
     int max_q = 0, max_qa = 0, max_cq = 0, max_ld = 0, max_e = 0;
     bool f32 = false;                  // number format of the projections and the key cache
@@ -887,6 +888,7 @@ void Model::alloc_runtime_layered() {
         L.sel = dalloc<int32_t>(cap * (size_t)L.max_top);
         L.srt = dalloc<int32_t>(cap * (size_t)L.max_top);
         L.off = dalloc<int32_t>((size_t)L.max_E + 1);
+        L.Z = dalloc<float>(cap * (size_t)L.max_E);
     }
     if (!L.f32) {
         int max_k = std::max({(int)W, L.max_o, L.max_ff, L.max_cq, L.max_sff}), dense_ff = L.max_sff;
@@ -1093,10 +1095,15 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
         if (W % 4 == 0 && L.embed_scale == 1.f) launch_embed_rows(embed, d_ids, L.X, T, W, V, s);
         else launch_lay_embed_rows(embed, d_ids, L.X, T, W, V, s, L.embed_scale);
         // the residual update of a finished sublayer waits for the next norm: decode steps run both in one launch
-        struct { const float* y = nullptr; const float* w = nullptr; const float* wsel = nullptr; int top = 0; } pend;
+        struct { const float* y = nullptr; const float* w = nullptr; const float* wsel = nullptr; int top = 0; int sel_top = 0, n_real = -1; } pend;
         auto flush_post = [&]() {
-            if (pend.y) launch_lay_post_norm(L.X, pend.y, pend.w, L.mult, cfg.eps, T, W, pend.wsel, pend.top, s);
-            pend.y = nullptr;
+            if (pend.y) {
+                // identity experts: their rows are the sublayer's input, which for this update is the residual itself (a thread reads
+                // an element of x before it writes it, and touches no other)
+                if (pend.n_real >= 0) launch_lay_post_norm(L.X, pend.y, pend.w, L.mult, cfg.eps, T, W, pend.wsel, pend.top, s, L.sel, pend.sel_top, pend.n_real, L.X);
+                else launch_lay_post_norm(L.X, pend.y, pend.w, L.mult, cfg.eps, T, W, pend.wsel, pend.top, s);
+            }
+            pend.y = nullptr; pend.n_real = -1;
         };
         auto post_norm = [&](const float* y, const float* w_, const float* wsel, int top) {
             flush_post();
@@ -1273,7 +1280,9 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                         if (L.fused_prep) {
                             launch_lay_qk_prep(L.P, w.in_rows, sw.q_off, sw.k_off, sw.v_off, H, G, d, e, sd.qk_norm ? sw.q_norm : nullptr,
                                                sd.qk_norm ? sw.k_norm : nullptr, cfg.eps, sd.rot.dims, sd.rot.half, sd.rot.dims > 0 ? sw.rot_freq : nullptr,
-                                               sw.rot_mag, kv_pool + sw.k_pool_off, kv_pool + sw.v_pool_off, kv_mode, d_bt, d_segs, d_rowseg, T, page, s);
+                                               sw.rot_mag, kv_pool + sw.k_pool_off, kv_pool + sw.v_pool_off, kv_mode, d_bt, d_segs, d_rowseg, T, page, s,
+                                               all_decode ? (int)sd.pool : 0, sw.pool_rows, all_decode && sd.pool > 0 ? kv_pool + sw.pk_pool_off : nullptr,
+                                               all_decode && sd.pool > 0 ? kv_pool + sw.pv_pool_off : nullptr);
                         } else {               // the same from the single operations
                             if (sd.qk_norm) {
                                 launch_lay_rms_cols(L.P, w.in_rows, sw.q_off, H * d, sw.q_norm, L.P + sw.q_off, w.in_rows, T, cfg.eps, s);
@@ -1288,7 +1297,7 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                             launch_lay_k_append(L.P, w.in_rows, sw.k_off, kv_pool + sw.k_pool_off, kv_mode, d_bt, d_segs, d_rowseg, T, G, d, page, s);
                             launch_lay_k_append(L.P, w.in_rows, sw.v_off, kv_pool + sw.v_pool_off, kv_mode, d_bt, d_segs, d_rowseg, T, G, e, page, s);
                         }
-                        if (sd.pool > 0)
+                        if (sd.pool > 0 && !(L.fused_prep && all_decode))
                             launch_lay_pool_append(kv_pool + sw.k_pool_off, kv_pool + sw.pk_pool_off, d, kv_pool + sw.v_pool_off, kv_pool + sw.pv_pool_off, e,
                                                    kv_mode, d_bt, d_segs, d_rowseg, T, G, page, (int)sd.pool, sw.pool_rows, s);
                         run_attention(sd, sw, L.P, w.in_rows, sw.q_off, 0, d, e, L.O + sw.o_col, ocols, sd.side_scale);
@@ -1317,7 +1326,7 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                 } else if (sp.mlp == LMLP_MOE) {
                     flush_post();
                     const int outs = sp.experts + sp.router.identity, slots = sp.top + (sp.shared_ff > 0 ? 1 : 0);
-                    launch_lay_router(L.X, w.router, L.sel, L.wsel, T, W, outs, sp.top, s, &sp.router, w.correction, slots);
+                    launch_lay_router(L.X, w.router, L.sel, L.wsel, T, W, outs, sp.top, s, &sp.router, w.correction, slots, L.Z);
                     launch_lay_moe_plan(L.sel, L.off, L.srt, T * sp.top, outs, s, sp.top, slots);
                     LGemmArgs gu;
                     gu.A = L.X; gu.lda = W; gu.a_idx = L.srt; gu.a_div = slots;
@@ -1328,7 +1337,6 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                     dn.A = L.HH; dn.lda = sp.ff; dn.W = w.down; dn.w_stride = (size_t)W * sp.ff;
                     dn.C = L.YS; dn.ldc = W; dn.c_idx = L.srt; dn.M = T; dn.N = W; dn.K = sp.ff; dn.grp_off = L.off;
                     lay_gemm(*this, L, dn, sp.experts, s);
-                    if (sp.router.identity > 0) launch_lay_moe_identity(L.sel, L.X, L.YS, T, W, sp.top, slots, sp.experts, s);
                     if (sp.shared_ff > 0) {        // the expert every token uses: row `top` of the token's rows, weight 1
                         LGemmArgs su;
                         su.A = L.X; su.lda = W; su.W = w.sh_gate; su.W2 = w.sh_up; su.C = L.HS; su.ldc = sp.shared_ff; su.M = T; su.N = sp.shared_ff;
@@ -1340,6 +1348,7 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                         lay_gemm(*this, L, sdn, 1, s);
                     }
                     post_norm(L.YS, w.norm2b, L.wsel, slots);
+                    if (sp.router.identity > 0) { pend.sel_top = sp.top; pend.n_real = sp.experts; }      // identity rows are taken in the combine
                 }
             } else {
             norm_canon(w.norm1, w.canon1, w.c1_off);
@@ -1376,7 +1385,7 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                     lay_gemm(*this, L, dn, 1, s);
                     post_norm(L.Y, w.norm2b, nullptr, 0);
                 } else {
-                    launch_lay_router(L.Hc, w.router, L.sel, L.wsel, T, W, sp.experts, sp.top, s);
+                    launch_lay_router(L.Hc, w.router, L.sel, L.wsel, T, W, sp.experts, sp.top, s, nullptr, nullptr, 0, L.Z);
                     launch_lay_moe_plan(L.sel, L.off, L.srt, T * sp.top, sp.experts, s);
                     LGemmArgs gu;
                     gu.A = L.Hc; gu.lda = W; gu.a_idx = L.srt; gu.a_div = sp.top;
