@@ -6,7 +6,7 @@ from tests.korupel_util import bf16_round, tokens, write_checkpoint  # noqa: F40
 
 def left(heads=4, kv_heads=2, dim=16, vdim=8, size=20, pool=6, scale=None, dims=None, base=10000.0, scaling="default"):
     if scaling == "default":
-        scaling = dict(factor=4.0, low=1.0, high=4.0, original=64)
+        scaling = dict(factor=3.0, low=1.0, high=5.0, original=64)
     rot = dict(base=base, dims=dim if dims is None else dims)
     if scaling is not None:
         rot["scaling"] = scaling
@@ -14,7 +14,7 @@ def left(heads=4, kv_heads=2, dim=16, vdim=8, size=20, pool=6, scale=None, dims=
                 mask=dict(size=size, pool=pool), rot=rot)
 
 
-def right(heads=2, dim=8, vdim=12, gate_cap=15.0):
+def right(heads=2, dim=8, vdim=12, gate_cap=12.0):
     return dict(heads=heads, dim=dim, vdim=vdim, gate_cap=gate_cap)
 
 

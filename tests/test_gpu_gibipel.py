@@ -297,6 +297,8 @@ OTHER = {
     "wide heads": U.config([U.layer(U.left(heads=2, kv_heads=1, dim=160, vdim=96, size=30, pool=8, scale=0.05, dims=64), U.right(heads=1, dim=144, vdim=48), None)],
                            width=72),
     "no window reached, no blocks": U.config([U.layer(U.left(size=500, pool=0), U.right(), U.moe())]),
+    "more router outputs than a wave has lanes": U.config(
+        [U.layer(U.left(), U.right(), U.moe(experts=70, top=6, ff=8, identity=2, groups=8, keep=3, shared=16))], width=32),
 }
 
 
@@ -484,11 +486,11 @@ def _drawn_config(seed):
     pick = lambda *xs: xs[rs.randint(len(xs))]
     width, layers = pick(96, 128, 192, 256, 320), []
     for _ in range(rs.randint(2, 6)):
-        kvh, dim = pick(1, 2, 4), pick(16, 24, 32, 64, 96)
+        kvh, dim = pick(1, 2, 4), pick(16, 24, 32, 64, 80)
         dims = pick(dim, dim // 2, dim // 4 * 2)
         scaling = pick(None, dict(factor=pick(2.0, 8.0), low=pick(1.0, 2.0), high=pick(4.0, 8.0), original=pick(32, 128, 2048)))
-        lf = U.left(heads=kvh * pick(1, 2, 3), kv_heads=kvh, dim=dim, vdim=pick(16, 32, 48, 96), size=pick(17, 40, 64, 72, 128), pool=pick(3, 8, 12, 16, 64),
-                    scale=pick(0.1, 0.2), dims=dims, base=pick(100.0, 10000.0, 250000.0), scaling=scaling)
+        lf = U.left(heads=kvh * pick(1, 2, 3), kv_heads=kvh, dim=dim, vdim=pick(16, 32, 48, 112), size=pick(17, 40, 64, 80, 128), pool=pick(3, 8, 10, 16, 64),
+                    scale=pick(0.1, 0.2), dims=dims, base=pick(100.0, 10000.0, 500000.0), scaling=scaling)
         rg = U.right(heads=pick(1, 2, 4), dim=pick(8, 16, 32, 64), vdim=pick(16, 32, 64, 72), gate_cap=pick(5.0, 15.0, 30.0))
         mlp = None
         if rs.rand() < 0.8:
