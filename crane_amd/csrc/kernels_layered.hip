@@ -877,10 +877,14 @@ __device__ __forceinline__ void lay_block_mean(const void* __restrict__ src, voi
     for (int i = threadIdx.x; i < G * n; i += 256) {
         const int g = i / n, c = i - g * n;
         float sum = 0.f;
+        // page by page: one table look-up, then rows at a fixed stride, so that several loads are in flight; the sum keeps position order
+        for (int j0 = b * pool; j0 <= pos;) {
+            const int j1 = min(pos + 1, (j0 / page + 1) * page);
+            const size_t at = (((size_t)bt[bt_off + j0 / page] * G + g) * page + (size_t)(j0 % page)) * n + c;
 #pragma unroll 8
-        for (int j = b * pool; j <= pos; ++j) {
-            const size_t at = (((size_t)bt[bt_off + j / page] * G + g) * page + (size_t)(j % page)) * n + c;
-            sum += KVT == KV_F32 ? ((const float*)src)[at] : bf16_to_f32(((const uint16_t*)src)[at]);
+            for (int j = 0; j < j1 - j0; ++j)
+                sum += KVT == KV_F32 ? ((const float*)src)[at + (size_t)j * n] : bf16_to_f32(((const uint16_t*)src)[at + (size_t)j * n]);
+            j0 = j1;
         }
         const size_t dst = (((size_t)bt[bt_off + lpg] * G + g) * pool_rows + idx) * n + c;
         if (KVT == KV_F32) ((float*)dstp)[dst] = sum * inv;
