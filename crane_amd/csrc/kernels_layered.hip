@@ -24,6 +24,12 @@ __device__ __forceinline__ float lay_act(float v, int act, float param = 1.f) {
         default: return v;
     }
 }
+// capped gated product: g = min(g, cap), u = clamp(u, -cap, cap): g sigmoid(1.702 g) (u + 1)
+__device__ __forceinline__ float lay_capglu(float g, float u, float cap) {
+    g = fminf(g, cap);
+    u = fminf(fmaxf(u, -cap), cap);
+    return g / (1.f + expf(-1.702f * g)) * (u + 1.f);
+}
 
 // sum over the block (blockDim.x a multiple of 64, every thread calls); red: >= blockDim.x / 64 floats of LDS
 __device__ __forceinline__ float block_sum(float v, float* red) {
@@ -208,7 +214,7 @@ __global__ __launch_bounds__(256) void lay_rms_gate_kernel(const float* __restri
     for (int c = threadIdx.x; c < N; c += 256) { const float v = orow[c]; ss += v * v; }
     ss = block_sum(ss, red);
     const float rs = 1.f / sqrtf(ss / (float)N + eps);
-    for (int c = threadIdx.x; c < N; c += 256) out[(size_t)r * N + c] = orow[c] * rs * w[c] * gate[(size_t)r * ldg + c];
+    for (int c = threadIdx.x; c < N; c += 256) out[(size_t)r * N + c] = orow[c] * rs * w[c] * (gate ? gate[(size_t)r * ldg + c] : 1.f);
 }
 // the same with the root mean square over groups of `group` columns: one wave per group
 __global__ __launch_bounds__(256) void lay_rms_gate_group_kernel(const float* __restrict__ o, const float* __restrict__ gate, int ldg,
@@ -223,7 +229,7 @@ __global__ __launch_bounds__(256) void lay_rms_gate_group_kernel(const float* __
         ss = wave_sum(ss);
         const float rs = 1.f / sqrtf(ss / (float)group + eps);
         for (int c = lane; c < group; c += 64)
-            out[(size_t)r * N + (size_t)g * group + c] = og[c] * rs * w[shared_w ? c : g * group + c] * gate[(size_t)r * ldg + (size_t)g * group + c];
+            out[(size_t)r * N + (size_t)g * group + c] = og[c] * rs * w[shared_w ? c : g * group + c] * (gate ? gate[(size_t)r * ldg + (size_t)g * group + c] : 1.f);
     }
 }
 void launch_lay_rms_gate(const float* o, const float* gate, int ldg, const float* w, float* out, int T, int N, float eps, hipStream_t s,
@@ -532,7 +538,7 @@ __device__ __forceinline__ bool lg_tile(const LGemmArgs& a, LgTile& t) {
 
 __device__ __forceinline__ void lg_store(const LGemmArgs& a, size_t coff, int p, int n, float v, float v2, bool dual) {
     if (a.bias) v += a.bias[n];
-    if (dual) v = lay_act(v, a.act) * v2;
+    if (dual) v = a.act == LACT_CAPGLU ? lay_capglu(v, v2, a.act_param) : lay_act(v, a.act) * v2;
     else v = lay_act(v, n < a.act_split ? a.act : a.act2, a.act_param);
     if (a.mul) v *= a.mul[(size_t)p * a.ldm + coff + n];
     const size_t row = a.c_idx ? (size_t)a.c_idx[p] : (size_t)p;
@@ -547,13 +553,19 @@ __global__ __launch_bounds__(256) void lgemm_f32_kernel(LGemmArgs a) {
     __shared__ float Bs[BK][LG_BN + 4];
     __shared__ float B2s[DUAL ? BK : 1][LG_BN + 4];
     __shared__ int arow[LG_BM];
+    __shared__ float ascl[LG_BM];
     LgTile t;
     if (!lg_tile(a, t)) return;
     const int tid = threadIdx.x;
     if (tid < LG_BM) {
         int ar = -1;
-        if (tid < t.rows) { const int p = t.p0 + tid; ar = a.a_idx ? a.a_idx[p] / a.a_div : p; }
-        arow[tid] = ar;
+        float sc = 1.f;
+        if (tid < t.rows) {
+            const int p = t.p0 + tid;
+            ar = a.a_idx ? a.a_idx[p] / a.a_div : p;
+            if (a.a_scale) sc = a.a_scale[a.a_idx[p]];
+        }
+        arow[tid] = ar; ascl[tid] = sc;
     }
     __syncthreads();
     const int ty = tid >> 4, tx = tid & 15;
@@ -562,7 +574,7 @@ __global__ __launch_bounds__(256) void lgemm_f32_kernel(LGemmArgs a) {
         for (int i = 0; i < 4; ++i) {
             const int idx = tid + i * 256, r = idx >> 4, kk = idx & 15, k = k0 + kk;
             const int ar = arow[r];
-            As[kk][r] = (ar >= 0 && k < a.K) ? t.A[(size_t)ar * a.lda + k] : 0.f;
+            As[kk][r] = (ar >= 0 && k < a.K) ? t.A[(size_t)ar * a.lda + k] * ascl[r] : 0.f;
             const int n = t.n0 + r;
             const bool ok = n < a.N && k < a.K;
             Bs[kk][r] = ok ? bf16_to_f32(t.W[(size_t)n * a.K + k]) : 0.f;
@@ -602,13 +614,19 @@ __global__ __launch_bounds__(256) void lgemm_bf16_kernel(LGemmArgs a) {
     __shared__ __attribute__((aligned(16))) uint16_t Bs[LG_BN][LDS_K];
     __shared__ __attribute__((aligned(16))) uint16_t B2s[DUAL ? LG_BN : 1][LDS_K];
     __shared__ int arow[LG_BM];
+    __shared__ float ascl[LG_BM];
     LgTile t;
     if (!lg_tile(a, t)) return;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     if (tid < LG_BM) {
         int ar = -1;
-        if (tid < t.rows) { const int p = t.p0 + tid; ar = a.a_idx ? a.a_idx[p] / a.a_div : p; }
-        arow[tid] = ar;
+        float sc = 1.f;
+        if (tid < t.rows) {
+            const int p = t.p0 + tid;
+            ar = a.a_idx ? a.a_idx[p] / a.a_div : p;
+            if (a.a_scale) sc = a.a_scale[a.a_idx[p]];
+        }
+        arow[tid] = ar; ascl[tid] = sc;
     }
     __syncthreads();
     const int wm = wave >> 1, wn = wave & 1;
@@ -627,6 +645,10 @@ __global__ __launch_bounds__(256) void lgemm_bf16_kernel(LGemmArgs a) {
                 v[0] = x0.x; v[1] = x0.y; v[2] = x0.z; v[3] = x0.w; v[4] = x1.x; v[5] = x1.y; v[6] = x1.z; v[7] = x1.w;
             } else {
                 for (int i = 0; i < 8; ++i) v[i] = (ar >= 0 && k + i < a.K) ? t.A[(size_t)ar * a.lda + k + i] : 0.f;
+            }
+            if (a.a_scale) {
+                const float sc = ascl[lr];
+                for (int i = 0; i < 8; ++i) v[i] *= sc;
             }
             u32x4 pk;
             pk.x = pack_bf16x2(v[0], v[1]); pk.y = pack_bf16x2(v[2], v[3]); pk.z = pack_bf16x2(v[4], v[5]); pk.w = pack_bf16x2(v[6], v[7]);
@@ -697,10 +719,12 @@ __global__ __launch_bounds__(256) void lgemv_kernel(LGemmArgs a) {
     if (n0 >= a.N) return;
     const int n1 = min(n0 + 1, a.N - 1);                 // odd N: the second column repeats the first and is not stored
     size_t ar[LV_MAXM];
+    float asc[LV_MAXM];
 #pragma unroll
     for (int r = 0; r < LV_MAXM; ++r) {
         const int p = base + min(r, rows - 1);
         ar[r] = (size_t)(a.a_idx ? a.a_idx[p] / a.a_div : p) * a.lda;
+        asc[r] = a.a_scale ? a.a_scale[a.a_idx[p]] : 1.f;
     }
     float acc[2][LV_MAXM] = {}, acc2[2][LV_MAXM] = {};
     const int K = a.K;
@@ -716,6 +740,10 @@ __global__ __launch_bounds__(256) void lgemv_kernel(LGemmArgs a) {
                 if (r < rows) {
                     const float4 xa = *(const float4*)(A + ar[r] + k), xb = *(const float4*)(A + ar[r] + k + 4);
                     float x[8] = {xa.x, xa.y, xa.z, xa.w, xb.x, xb.y, xb.z, xb.w};
+                    if (a.a_scale) {
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) x[i] *= asc[r];
+                    }
                     if (BF16) {
 #pragma unroll
                         for (int i = 0; i < 8; ++i) x[i] = bf16_round(x[i]);
@@ -739,7 +767,7 @@ __global__ __launch_bounds__(256) void lgemv_kernel(LGemmArgs a) {
 #pragma unroll
             for (int r = 0; r < LV_MAXM; ++r) {
                 if (r < rows) {
-                    float x = A[ar[r] + k];
+                    float x = A[ar[r] + k] * asc[r];
                     if (BF16) x = bf16_round(x);
                     acc[0][r] = fmaf(w0, x, acc[0][r]); acc[1][r] = fmaf(w1, x, acc[1][r]);
                     if (DUAL) { acc2[0][r] = fmaf(v0, x, acc2[0][r]); acc2[1][r] = fmaf(v1, x, acc2[1][r]); }
@@ -774,13 +802,13 @@ void launch_lay_act_cols(float* C, int ldc, int M, int N, int act, int act2, int
 }
 // out = act(g) * u
 __global__ __launch_bounds__(256) void lay_act_mul_kernel(const float* __restrict__ g, const float* __restrict__ u, float* __restrict__ out,
-                                                          size_t n, int act) {
+                                                          size_t n, int act, float param) {
     const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (i < n) out[i] = lay_act(g[i], act) * u[i];
+    if (i < n) out[i] = act == LACT_CAPGLU ? lay_capglu(g[i], u[i], param) : lay_act(g[i], act) * u[i];
 }
-void launch_lay_act_mul(const float* g, const float* u, float* out, size_t n, int act, hipStream_t s) {
+void launch_lay_act_mul(const float* g, const float* u, float* out, size_t n, int act, hipStream_t s, float param) {
     if (n == 0) return;
-    hipLaunchKernelGGL(lay_act_mul_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, g, u, out, n, act);
+    hipLaunchKernelGGL(lay_act_mul_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, g, u, out, n, act, param);
 }
 // rows of f32 -> bfloat16 (round to nearest even): the A operand of the shared matrix-core GEMM
 __global__ __launch_bounds__(256) void lay_round_rows_kernel(const float* __restrict__ x, int ldx, uint16_t* __restrict__ out, int K) {
@@ -862,7 +890,8 @@ __device__ __forceinline__ LaRow la_row(const LAttnArgs& a, const LaySegDev& sg,
         const int j = v < front ? v : main_lo + (v - front);
         const size_t row = ((size_t)a.bt[sg.bt_off + j / a.page] * a.G + g) * a.page + (size_t)(j % a.page);
         r.k = (const char*)a.kpool + row * a.d * ESZ;
-        r.v = a.vpool ? (const char*)a.vpool + row * a.e * ESZ : nullptr;
+        const size_t vrow = a.v_div > 1 ? ((size_t)a.bt[sg.bt_off + j / a.page] * (a.G / a.v_div) + g / a.v_div) * a.page + (size_t)(j % a.page) : row;
+        r.v = a.vpool ? (const char*)a.vpool + vrow * a.e * ESZ : nullptr;
     }
     return r;
 }
@@ -926,10 +955,15 @@ struct LQkPrepArgs {
     // pool > 0: every portion of the pass is ONE token, and a row that closes a block of `pool` positions also writes the block's mean
     // rows (the other positions of the block were cached by earlier passes; its own by this block)
     int pool, pool_rows; void *pk_pool, *pv_pool;
+    // head_norm: every head over its own root mean square, weights [d] shared by the heads (head_rs: a place per head, H + G of them);
+    // Gv value heads; qt_coef != 0: the query times 1 + qt_coef ln(floor((pos + 1) / qt_every) + 1)
+    int head_norm, Gv; float qt_coef; int qt_every;
 };
+constexpr int LQK_MAX_HEADS = 1024;
 template <int KVT>
 __global__ __launch_bounds__(256) void lay_qk_prep_kernel(LQkPrepArgs a) {
     __shared__ float red[4];
+    __shared__ float head_rs[LQK_MAX_HEADS];
     const int r = blockIdx.x, tid = threadIdx.x;
     const LaySegDev sg = a.segs[a.rowseg[r]];
     const int pos = sg.start_pos + (r - sg.row0);
@@ -937,16 +971,26 @@ __global__ __launch_bounds__(256) void lay_qk_prep_kernel(LQkPrepArgs a) {
     float* k = a.proj + (size_t)r * a.ldp + a.k_off;
     const int nq = a.H * a.d, nk = a.G * a.d;
     float rq = 1.f, rk = 1.f;
-    if (a.qn) {
+    if (a.head_norm) {                     // one wave per head: its own root mean square
+        for (int v = tid >> 6; v < a.H + a.G; v += 4) {
+            const float* x = v < a.H ? q + v * a.d : k + (v - a.H) * a.d;
+            float ss = 0.f;
+            for (int i = tid & 63; i < a.d; i += 64) ss += x[i] * x[i];
+            ss = wave_sum(ss);
+            if ((tid & 63) == 0) head_rs[v] = 1.f / sqrtf(ss / (float)a.d + a.eps);
+        }
+        __syncthreads();
+    } else if (a.qn) {
         float ss = 0.f;
         for (int i = tid; i < nq; i += 256) { const float v = q[i]; ss += v * v; }
         rq = 1.f / sqrtf(block_sum(ss, red) / (float)nq + a.eps);
     }
-    if (a.kn) {
+    if (a.kn && !a.head_norm) {
         float ss = 0.f;
         for (int i = tid; i < nk; i += 256) { const float v = k[i]; ss += v * v; }
         rk = 1.f / sqrtf(block_sum(ss, red) / (float)nk + a.eps);
     }
+    const float qt = a.qt_coef != 0.f ? 1.f + a.qt_coef * logf((float)((pos + 1) / a.qt_every) + 1.f) : 1.f;
     const int pg = a.bt[sg.bt_off + pos / a.page];
     const size_t prow = (size_t)pg * a.G * a.page + (size_t)(pos % a.page);       // + g * page: the cached row of key head g
     // a thread owns both elements of a pair (or one element past the rotated part)
@@ -958,12 +1002,16 @@ __global__ __launch_bounds__(256) void lay_qk_prep_kernel(LQkPrepArgs a) {
         const int hh = isq ? v : v - a.H;
         float* x = (isq ? q : k) + hh * a.d;
         const float* w = isq ? a.qn : a.kn;
-        const float rs = isq ? rq : rk;
+        const float rs = (a.head_norm ? head_rs[v] : (isq ? rq : rk)) * (isq ? qt : 1.f);
         int i0, i1 = -1;
         if (i < hd) { i0 = a.half ? i : 2 * i; i1 = a.half ? i + hd : 2 * i + 1; }
         else i0 = a.dims + (i - hd);
         float x0 = x[i0] * rs, x1 = i1 >= 0 ? x[i1] * rs : 0.f;
-        if (w) { x0 *= w[hh * a.d + i0]; if (i1 >= 0) x1 *= w[hh * a.d + i1]; }
+        if (w) {
+            const int wo = a.head_norm ? 0 : hh * a.d;
+            x0 *= w[wo + i0];
+            if (i1 >= 0) x1 *= w[wo + i1];
+        }
         if (i1 >= 0) {
             float sn, cs;
             sincosf(fpos * a.freq[i], &sn, &cs);
@@ -980,9 +1028,10 @@ __global__ __launch_bounds__(256) void lay_qk_prep_kernel(LQkPrepArgs a) {
     }
     if (a.vpool) {
         const float* vv = a.proj + (size_t)r * a.ldp + a.v_off;
-        for (int i = tid; i < a.G * a.e; i += 256) {
+        const size_t vrow = (size_t)pg * a.Gv * a.page + (size_t)(pos % a.page);
+        for (int i = tid; i < a.Gv * a.e; i += 256) {
             const int g = i / a.e, c = i - g * a.e;
-            const size_t dst = (prow + (size_t)g * a.page) * a.e + c;
+            const size_t dst = (vrow + (size_t)g * a.page) * a.e + c;
             if (KVT == KV_F32) ((float*)a.vpool)[dst] = vv[i];
             else ((uint16_t*)a.vpool)[dst] = f32_to_bf16(vv[i]);
         }
@@ -997,10 +1046,12 @@ __global__ __launch_bounds__(256) void lay_qk_prep_kernel(LQkPrepArgs a) {
 void launch_lay_qk_prep(float* proj, int ldp, int q_off, int k_off, int v_off, int H, int G, int d, int e, const float* qn, const float* kn,
                         float eps, int dims, bool half, const float* freq, float mag, void* kpool, void* vpool, int kvt, const int32_t* bt,
                         const LaySegDev* segs, const int32_t* rowseg, int T, int page, hipStream_t s, int pool, int pool_rows, void* pk_pool,
-                        void* pv_pool) {
+                        void* pv_pool, const LQkPrepExtra* extra) {
     if (T <= 0) return;
+    const LQkPrepExtra x = extra ? *extra : LQkPrepExtra();
     LQkPrepArgs a{proj, ldp, q_off, k_off, v_off, H, G, d, e, qn, kn, eps, freq ? dims : 0, half ? 1 : 0, freq, mag, kpool, vpool, bt, segs, rowseg, page,
-                  pk_pool ? pool : 0, pool_rows, pk_pool, pv_pool};
+                  pk_pool ? pool : 0, pool_rows, pk_pool, pv_pool, x.head_norm && H + G <= LQK_MAX_HEADS ? 1 : 0, x.Gv > 0 ? x.Gv : G, x.qt_coef,
+                  x.qt_every > 0 ? x.qt_every : 1};
     if (kvt == KV_F32) hipLaunchKernelGGL(lay_qk_prep_kernel<KV_F32>, dim3((unsigned)T), dim3(256), 0, s, a);
     else hipLaunchKernelGGL(lay_qk_prep_kernel<KV_BF16>, dim3((unsigned)T), dim3(256), 0, s, a);
 }
@@ -1437,8 +1488,11 @@ constexpr int LL_ES = 32;
 __device__ __forceinline__ float ll_ldec(const LLightArgs& a, int row, int head, int i) {
     return a.head_decay ? a.ldec[(size_t)row * a.ldd + head] : a.ldec[(size_t)row * a.ldd + (size_t)head * a.d + i];
 }
+__device__ __forceinline__ float ll_query(const LLightArgs& a, int row, int head, int i) {
+    return a.proj[(size_t)row * a.ldp + a.q_off + (size_t)(head / a.qk_rep) * a.d + i] * a.qscale;
+}
 __device__ __forceinline__ float ll_key(const LLightArgs& a, int row, int head, int i) {
-    const float k = a.proj[(size_t)row * a.ldp + a.k_off + (size_t)head * a.d + i];
+    const float k = a.proj[(size_t)row * a.ldp + a.k_off + (size_t)(head / a.qk_rep) * a.d + i];
     return a.kmul ? k * a.kmul[(size_t)row * a.ldd + head] : k;
 }
 __device__ __forceinline__ float ll_val(const LLightArgs& a, int row, int head, int c) {
@@ -1480,8 +1534,7 @@ __global__ __launch_bounds__(256) void lay_lightning_kernel(LLightArgs a, int C)
         __syncthreads();                   // S, pw ready; the previous chunk's q / k / v no longer read
         for (int idx = tid; idx < n * d; idx += 256) {
             const int t = idx / d, i = idx - t * d;
-            const size_t base = (size_t)(sg.row0 + t0 + t) * a.ldp + (size_t)head * d + i;
-            qs[idx] = a.proj[base + a.q_off] * a.qscale;
+            qs[idx] = ll_query(a, sg.row0 + t0 + t, head, i);
             ks[idx] = ll_key(a, sg.row0 + t0 + t, head, i);
             if (GT) bs[idx] = ll_ldec(a, sg.row0 + t0 + t, head, i);
         }
@@ -1650,8 +1703,7 @@ __global__ __launch_bounds__(256) void lay_light_chunk_out_kernel(LLightArgs a) 
     load_slice();
     for (int idx = tid; idx < n * d; idx += 256) {
         const int t = idx / d, i = idx - t * d;
-        const size_t base = (size_t)(sg.row0 + ch.y + t) * a.ldp + (size_t)head * d + i;
-        qs[idx] = a.proj[base + a.q_off] * a.qscale;
+        qs[idx] = ll_query(a, sg.row0 + ch.y + t, head, i);
         ks[t * ldk + i] = ll_key(a, sg.row0 + ch.y + t, head, i);
         if (GT) bs[t * ldk + i] = ll_ldec(a, sg.row0 + ch.y + t, head, i);
     }
@@ -1714,9 +1766,8 @@ __global__ __launch_bounds__(256) void lay_light_decode_kernel(LLightArgs a) {
     const int head = blockIdx.y, j0 = blockIdx.z * LL_ES, tid = threadIdx.x;
     const int j = tid & (LL_ES - 1), rg = tid >> 5;
     const float decay = GT ? 1.f : a.decay[head];
-    const size_t prow = (size_t)sg.row0 * a.ldp;
     for (int i = tid; i < d; i += 256) {
-        qk[i] = a.proj[prow + a.q_off + (size_t)head * d + i] * a.qscale;
+        qk[i] = ll_query(a, sg.row0, head, i);
         qk[256 + i] = ll_key(a, sg.row0, head, i);
         if (GT) qk[512 + i] = expf(ll_ldec(a, sg.row0, head, i));
     }

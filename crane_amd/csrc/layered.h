@@ -14,6 +14,15 @@
 //     half-split rotation with banded frequency stretching, sink), and a matrix memory with exponential input / forget gates
 //     (running-maximum stabiliser, normaliser vector); mixture-of-experts feed-forwards with a softmax router (choice by score +
 //     correction inside the best groups of neighbours, identity experts, a shared expert).
+//   Nevotar -- pre-norm layers (x += mixer(norm1 x), x += ff(norm2 x)) whose RMS norms work on equal consecutive parts of the
+//     vector; a layer may run on an earlier layer's tensors with a cache and state of its own; the logits come from the embedding
+//     table.  Mixers: differential attention (two causal softmax maps per head over the same values, the second taken off the first
+//     times a learned number, unit RMS per head; the query grows with the logarithm of its position), a gated linear recurrence
+//     whose forget gate also sets what is written (lower-bounded gates), and two mixers side by side: sliding-window attention with
+//     per-head query / key norm, partial half-split rotation and the heads' scores mixed by a matrix before the softmax, next to a
+//     state-space mixer (short causal convolution with bias and SiLU, one decay per head and token from a softplus step size, keys
+//     and queries shared by groups of heads, skip term, gate before a grouped norm).  Mixture-of-experts feed-forwards whose expert
+//     weight multiplies the expert's INPUT, with a capped gated activation, plus a shared expert.
 // The mechanisms are kernels with their constants as arguments (kernels_layered.hip); the per-layer plumbing and the step function
 // over mixed batches (prompt portions beside single decode tokens) are in model_layered.cpp.
 #pragma once
@@ -26,10 +35,12 @@
 namespace cm {
 
 // LMIX_SIDE: the mixers in LayerSpec::side run side by side on the layer's input; LMIX_MEMORY: matrix memory with exponential gates
-enum { LMIX_ATTN = 0, LMIX_LIGHTNING = 1, LMIX_LATENT = 2, LMIX_GLA = 3, LMIX_MEMORY = 4, LMIX_SIDE = 5 };
+// LMIX_HGRN: gated linear recurrence with k = 1 - forget gate; LMIX_SSM: state-space mixer (one decay per head and token)
+enum { LMIX_ATTN = 0, LMIX_LIGHTNING = 1, LMIX_LATENT = 2, LMIX_GLA = 3, LMIX_MEMORY = 4, LMIX_SIDE = 5, LMIX_HGRN = 6, LMIX_SSM = 7 };
 enum { LMLP_NONE = 0, LMLP_DENSE = 1, LMLP_MOE = 2 };
 // LACT_RELU2: max(v, 0)^2;  LACT_LOGSIG: act_param * ln(sigmoid(v)) (the logarithm of a decay sigmoid(v)^act_param)
-enum { LACT_NONE = 0, LACT_SILU = 1, LACT_SIGMOID = 2, LACT_GELU_TANH = 3, LACT_RELU2 = 4, LACT_LOGSIG = 5 };
+// LACT_CAPGLU (two-matrix products only): g = min(g, cap), u = clamp(u, -cap, cap): g sigmoid(1.702 g) (u + 1), cap = act_param
+enum { LACT_NONE = 0, LACT_SILU = 1, LACT_SIGMOID = 2, LACT_GELU_TANH = 3, LACT_RELU2 = 4, LACT_LOGSIG = 5, LACT_CAPGLU = 6 };
 // distance term taken off an attention score: none | r1 ln(1 + r2 (i - j)) | r1 (i - j)
 enum { LBIAS_NONE = 0, LBIAS_LOG = 1, LBIAS_LINEAR = 2 };
 // gate on the attention output: none | one value per head at g_off + head | one per element at g_off + head e + i
@@ -82,6 +93,17 @@ struct LayerSpec {
     int shared_ff = 0;                 // mixture of experts: inner size of the expert every token uses (0: none)
     std::vector<LayerSpec> side;       // LMIX_SIDE: the mixers, each scaled by its side_scale
     float side_scale = 1.f;
+    // attention: `maps` softmax maps per head over the same values (q and k hold maps * dim elements per head, map by map); two maps
+    // are combined as unit_rms(a1 - lambda a2) (1 - diff)
+    int maps = 1; float diff = 0.f;
+    float qt_coef = 0.f; long long qt_every = 0;   // attention: q times 1 + qt_coef ln(floor((p + 1) / qt_every) + 1) at position p (0: off)
+    bool talk = false;                 // attention: the heads' scores are mixed by a matrix [H][H] before mask and softmax
+    bool head_norm = false;            // attention: RMS norm of every query (key) head by itself, one weight vector [dim] for all heads
+    // state-space mixer: state size per head, groups of heads that share keys (B) and queries (C), convolution taps, parts of the output norm
+    int state = 0, groups = 1, conv = 0, norm_groups = 1;
+    bool scale_input = false;          // mixture of experts: the expert's weight multiplies its input (false: its output)
+    int expert_act = LACT_SILU; float limit = 0.f, shared_limit = 0.f;    // experts: activation of the gated product and its cap
+    int weights_of = -1;               // the layer runs on that earlier layer's tensors, with a cache and state of its own
 };
 
 // device-side weights of one layer (bf16 matrices [out, in], f32 vectors)
@@ -120,6 +142,14 @@ struct LayeredLayerW {
     float* correction = nullptr;                     // router: [outputs]
     uint16_t *sh_gate = nullptr, *sh_up = nullptr, *sh_down = nullptr;   // shared expert
     int o_col = 0;                                   // side mixers: first column of this mixer's heads in the joint output projection's input
+    float* talk = nullptr;                           // attention: [H][H] score mixing matrix
+    float lambda = 0.f;                              // two-map attention: the factor on the second map
+    float* lower = nullptr;                          // gated recurrence: [H d] lower bound of the forget gate
+    // state-space mixer: convolution [channels][taps] + bias, step-size bias [H], -exp(A_log) [H], skip factor [H]; columns of the
+    // projection row: z_off (gate) | x_off (x | B | C: the convolution's channels) | dt_off
+    float *conv_w = nullptr, *conv_b = nullptr, *dt_bias = nullptr, *a_neg = nullptr, *skip = nullptr;
+    int z_off = 0, x_off = 0, dt_off = 0;
+    size_t cv_off = 0;                               // the convolution's last taps - 1 inputs inside a slot of the conv pool (floats)
     std::vector<LayeredLayerW> side;
 };
 
@@ -142,13 +172,14 @@ struct LGemmArgs {
     // groups without grp_off (one product per head over all rows): group g reads A + g a_goff, writes C + g c_goff
     size_t a_goff = 0, c_goff = 0;
     const float* mul = nullptr; int ldm = 0;         // C[p][n] *= mul[p ldm + g c_goff + n] after the activation
+    const float* a_scale = nullptr;                  // with a_idx: the A row of output row p is multiplied by a_scale[a_idx[p]] (before any rounding)
 };
 // bf16 = true: A rounded to bfloat16, matrix cores, f32 accumulation; false: f32 FMA throughout.  Up to 8 rows (per group): the
 // streaming row kernel instead of tiles.
 void launch_lgemm(const LGemmArgs& a, bool bf16, int groups, hipStream_t s);
 
 void launch_lay_act_cols(float* C, int ldc, int M, int N, int act, int act2, int split, hipStream_t s, float param = 1.f);
-void launch_lay_act_mul(const float* g, const float* u, float* out, size_t n, int act, hipStream_t s);
+void launch_lay_act_mul(const float* g, const float* u, float* out, size_t n, int act, hipStream_t s, float param = 1.f);
 void launch_lay_round_rows(const float* x, int ldx, uint16_t* out, int M, int K, hipStream_t s);
 void launch_lay_embed_rows(const uint16_t* emb, const uint32_t* ids, float* x, int T, int W, int V, hipStream_t s, float scale = 1.f);
 void launch_lay_rms_rows(const float* x, const int32_t* rows, const float* w, float* out, int n_rows, int W, float eps, hipStream_t s);
@@ -203,6 +234,7 @@ struct LAttnArgs {
     // b pool + pool - 1 <= i - win; rows [n_pages][G][pool_rows][d] / [e] (lay_pool_append), in front of the window in the key walk
     long long pool = 0; const void* pk_pool = nullptr; const void* pv_pool = nullptr; int pool_rows = 0;
     float out_scale = 1.f;                           // factor on the output
+    int v_div = 1;                                   // v_div consecutive key heads share one value head: value pages [n_pages][G / v_div][page][e]
 };
 void launch_lay_k_append(const float* proj, int ldp, int k_off, void* kpool, int kvt, const int32_t* bt, const LaySegDev* segs,
                          const int32_t* rowseg, int T, int G, int d, int page, hipStream_t s);
@@ -211,6 +243,9 @@ void launch_lay_k_append(const float* proj, int ldp, int k_off, void* kpool, int
 // Keys [..][d] and -- vpool given -- values [..][e] in one launch.
 void launch_lay_pool_append(const void* kpool, void* pk_pool, int d, const void* vpool, void* pv_pool, int e, int kvt, const int32_t* bt,
                             const LaySegDev* segs, const int32_t* rowseg, int T, int G, int page, int pool, int pool_rows, hipStream_t s);
+// more of lay_qk_prep: head_norm -- every head is normed by itself with the weights qn / kn [d] (shared by the heads); Gv -- value
+// heads (0: as many as key heads); qt_coef / qt_every -- the query is multiplied by 1 + qt_coef ln(floor((p + 1) / qt_every) + 1)
+struct LQkPrepExtra { bool head_norm = false; int Gv = 0; float qt_coef = 0.f; int qt_every = 0; };
 // queries and keys of a pass on their way into attention, one launch: RMS norm over all query heads at once and over all key heads
 // at once (qn / kn: weights [H d] / [G d]; null: no norm), rotation by position (freq null: none), q back in place, keys -- and
 // values, vpool given -- into the pages.  pk_pool given (only when every portion of the pass is one token): the mean rows of a block that
@@ -218,7 +253,7 @@ void launch_lay_pool_append(const void* kpool, void* pk_pool, int d, const void*
 void launch_lay_qk_prep(float* proj, int ldp, int q_off, int k_off, int v_off, int H, int G, int d, int e, const float* qn, const float* kn,
                         float eps, int dims, bool half, const float* freq, float mag, void* kpool, void* vpool, int kvt, const int32_t* bt,
                         const LaySegDev* segs, const int32_t* rowseg, int T, int page, hipStream_t s, int pool = 0, int pool_rows = 0,
-                        void* pk_pool = nullptr, void* pv_pool = nullptr);
+                        void* pk_pool = nullptr, void* pv_pool = nullptr, const LQkPrepExtra* extra = nullptr);
 inline int lay_pool_rows(int page, long long pool) { return pool >= page ? 1 : (int)((page + pool - 1) / pool); }
 void launch_lay_attn(const LAttnArgs& a, int kvt, hipStream_t s);    // kvt: KV_BF16 | KV_F32
 bool lay_attn_fits(int d, int e, bool own_v);                         // sizes the kernel can hold in LDS and registers
@@ -248,6 +283,7 @@ struct LLightArgs {
     // k_t * kmul[t ldd + head].  ones_col: the last of the e value columns is the constant 1 (the projection row holds e - 1 per
     // head), so that the state's last column carries sum_s decay(s..t) k_s -- the normaliser of a matrix memory
     bool head_decay = false; const float* kmul = nullptr; bool ones_col = false;
+    int qk_rep = 1;              // qk_rep consecutive heads share one query / key vector: q and k hold H / qk_rep vectors of d
 };
 constexpr int LAY_LIGHT_CHUNK = 32;
 void launch_lay_lightning(const LLightArgs& a, hipStream_t s);
@@ -255,6 +291,39 @@ void launch_lay_lightning(const LLightArgs& a, hipStream_t s);
 // whole row) and group g's column c uses w[c] (weights shared by the groups) or w[g group + c] (shared_w false).
 void launch_lay_rms_gate(const float* o, const float* gate, int ldg, const float* w, float* out, int T, int N, float eps, hipStream_t s,
                          int group = 0, bool shared_w = false);
+
+// ---- kernels_layered_mix.hip ----
+// x[r] += sum_(k < nsum) y[(r nsum + k) W ..] (y null: nothing is added), then out[r] = x[rows ? rows[r] : r] in `groups` equal
+// consecutive parts, each over its own root mean square, times w (out null: the update alone).  rows and y exclude each other.
+void launch_lay_add_gnorm(float* x, const int32_t* rows, const float* y, int nsum, const float* w, float* out, int n_rows, int W, int groups,
+                          float eps, hipStream_t s);
+// two-map attention: a [T][2 H e] holds the maps' outputs, key head g's heads of map m at columns ((2 g + m) nrep + j) e; out[t][h e + i] =
+// unit_rms_e(a1 - lambda a2) * post
+void launch_lay_diff_combine(const float* a, float* out, int T, int H, int G, int e, float lambda, float post, float eps, hipStream_t s);
+// gated recurrence: z = proj[t][f_off + i] -> forget gate f = l + (1 - l) sigmoid(z); proj[t][f_off + i] <- 1 - f, ldec[t n + i] = ln f
+void launch_lay_hgrn_gates(float* proj, int ldp, int f_off, const float* lower, float* ldec, int T, int n, hipStream_t s);
+// causal convolution per channel with bias and activation: dst[t][c] = act(sum_j cw[c][j] src[t - taps + 1 + j][off + c] + cb[c]); inputs in
+// front of a portion come from the sequence's tail in conv_pool ([taps - 1][C], oldest first).  H > 0: per head also the state-space
+// step dt = softplus(src[t][dt_off + h] + dt_bias[h]) -> kmul[t H + h] = dt, ldec[t H + h] = a_neg[h] dt.  tail_too (every portion of
+// the pass is one token): the thread of a channel also shifts its tail; otherwise launch_lay_conv_tail follows.
+struct LConvArgs {
+    const float* src; int lds, off, C; float* dst; int ldd; const float *cw, *cb; int taps, act;
+    float* conv_pool; size_t slot_stride, cv_off; const LaySegDev* segs; const int32_t* rowseg;
+    int H = 0, dt_off = 0; const float *dt_bias = nullptr, *a_neg = nullptr; float *ldec = nullptr, *kmul = nullptr;
+    bool tail_too = false;
+};
+void launch_lay_conv_act(const LConvArgs& a, int T, hipStream_t s);
+void launch_lay_conv_tail(const LConvArgs& a, int nseg, hipStream_t s);
+// state-space output: y = (o[t][h e + i] + skip[h] x[t][x_off + h e + i]) silu(z[t][z_off + h e + i]), RMS norm in norm_groups equal
+// parts, times w times out_scale -> out[t ldo + ..]
+void launch_lay_ssm_out(const float* o, const float* x, int ldx, int x_off, const float* z, int ldz, int z_off, const float* skip, const float* w,
+                        float* out, int ldo, int T, int H, int e, int norm_groups, float eps, float out_scale, hipStream_t s);
+// softmax attention whose heads' scores are mixed before mask and softmax: score'_h = sum_g talk[h H + g] score_g.  A block owns
+// some positions of one sequence with ALL heads; uses of LAttnArgs: proj / q_off, out / ldo / out_scale, kpool, vpool (needed), bt, segs,
+// H, G, d, e, page, scale, win.  nseg segments, portions of up to max_n tokens; nsplit > 1 (only when max_n == 1): the keys are dealt
+// to nsplit blocks and merged, part_o / part_ml hold nseg nsplit H rows.
+void launch_lay_attn_talk(const LAttnArgs& a, const float* talk, int nseg, int max_n, int kvt, hipStream_t s);
+bool lay_attn_talk_fits(int H, int G, int d, int e);
 
 // router: z = h . Wr^T in f32 over E outputs, scores by rs (sigmoid of each / softmax over all), the `top` largest choice scores
 // (score + correction, inside the best groups; lowest index first among equals) -> sel [T top], wsel [T slots] = their scores

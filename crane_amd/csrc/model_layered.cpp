@@ -28,6 +28,12 @@ struct Layered {
     // Gibipel: a sublayer reads the residual itself and a one-number norm sits on its output; embedding and logits are scaled
     bool post_only = false;
     float embed_scale = 1.f, logit_scale = 1.f;
+    // Nevotar: x += mixer(norm1 x), x += ff(norm2 x); the norms work on norm_groups equal parts of the vector; the logits come from the
+    // embedding table
+    bool pre_norm = false;
+    int norm_groups = 1;
+    int max_conv = 0;                  // widest convolution of a state-space mixer (channels)
+    float* XB = nullptr;               // [cap][max_conv] convolved and activated channels
     int max_mh = 0, max_sff = 0, max_slots = 1;   // matrix-memory heads, shared expert size, rows per token of an expert combine
     float* Z = nullptr;                // router logits [cap][most outputs]
     float *KM = nullptr, *MR = nullptr, *HS = nullptr;   // matrix memory: key factor and running maximum per token and head; shared expert's inner rows
@@ -86,7 +92,7 @@ static void lay_gemm(Model& m, Layered& L, const LGemmArgs& g, int groups, hipSt
         bool ok = launch_gemm(a, GEPI_STORE, s);
         if (ok && g.W2) { a.W = g.W2; a.C = L.G2; ok = launch_gemm(a, GEPI_STORE, s); }
         if (ok) {
-            if (g.W2) launch_lay_act_mul(L.G1, L.G2, g.C, (size_t)g.M * g.N, g.act, s);
+            if (g.W2) launch_lay_act_mul(L.G1, L.G2, g.C, (size_t)g.M * g.N, g.act, s, g.act_param);
             else launch_lay_act_cols(g.C, g.ldc, g.M, g.N, g.act, g.act2, g.act_split, s, g.act_param);
             return;
         }
@@ -121,6 +127,7 @@ static void parse_mlp(const cmjson::Value* ml, LayerSpec& sp, bool moe_ok) {
         const cmjson::Value* rt = ml->get("router");
         if (!ex || !rt) throw CmError(CM_ERR_IO, "config.json: moe without expert / router");
         sp.ff = (int)ex->integer("ff", 0);
+        sp.limit = (float)ex->number("limit", 0.0);
         sp.experts = (int)rt->integer("experts", 0);
         sp.top = (int)rt->integer("top", 0);
         sp.router.identity = (int)rt->integer("identity", 0);
@@ -137,6 +144,7 @@ static void parse_mlp(const cmjson::Value* ml, LayerSpec& sp, bool moe_ok) {
         if (const cmjson::Value* sh = ml->get("shared"))
             if (sh->kind == cmjson::Value::Obj) {
                 sp.shared_ff = (int)sh->integer("ff", 0);
+                sp.shared_limit = (float)sh->number("limit", 0.0);
                 if (sp.shared_ff <= 0) throw CmError(CM_ERR_IO, "config.json: shared.ff");
             }
     } else throw CmError(CM_ERR_UNSUPPORTED, "mlp.kind '" + kind + "' not implemented");
@@ -310,36 +318,146 @@ static void parse_gibipel_layer(const cmjson::Value& e, LayerSpec& sp) {
     sp.router.softmax = true; sp.router.correction = true; sp.router.normalise = true;
 }
 
+// softmax attention sizes shared by Nevotar's two attention kinds
+static void parse_attn_sizes(const cmjson::Value& mx, LayerSpec& a) {
+    a.mixer = LMIX_ATTN;
+    a.heads = (int)mx.integer("heads", 0);
+    a.kv_heads = (int)mx.integer("kv_heads", a.heads);
+    a.dim = (int)mx.integer("dim", 0);
+    a.vdim = (int)mx.integer("vdim", a.dim);
+    need(a.heads > 0 && a.dim > 0 && a.vdim > 0 && a.kv_heads > 0 && a.heads % a.kv_heads == 0, "attention sizes");
+    a.scale = (float)mx.number("scale", 1.0 / std::sqrt((double)a.dim));
+    a.win = 1ll << 40; a.keep = 0;
+    a.bias = LBIAS_NONE; a.gate = LGATE_NONE; a.sink = false; a.own_v = true; a.qkv_bias = true;
+}
+
+// Nevotar: layer types "attention" (two softmax maps per head: "diff", "q_temp": {"coef", "every"}), "hgrn2", and "parallel" =
+// "mixer": {"left": window attention with "rot": {"base", "dims"}, "mask": {"size"} and mixed heads, "right": state-space mixer
+// {"heads", "vdim", "state", "groups", "conv", "norm_groups"}, "left_scale", "right_scale"}; "mlp": mixture of experts whose weights
+// multiply the experts' inputs ("expert": {"ff", "limit"}, "shared": {"ff", "limit"}); "weights_of": the layer whose tensors it uses
+static void parse_nevotar_layer(const cmjson::Value& e, LayerSpec& sp, const std::vector<LayerSpec>& before) {
+    const std::string type = e.string("type", "");
+    const cmjson::Value* mx = e.get("mixer");
+    need(mx && mx->kind == cmjson::Value::Obj, "layer without mixer");
+    if (type == "attention") {
+        parse_attn_sizes(*mx, sp);
+        sp.maps = 2;
+        sp.diff = (float)mx->number("diff", 0.0);
+        if (const cmjson::Value* qt = mx->get("q_temp"))
+            if (qt->kind == cmjson::Value::Obj) {
+                sp.qt_coef = (float)qt->number("coef", 0.0);
+                sp.qt_every = qt->integer("every", 1);
+                need(sp.qt_every > 0 && sp.qt_every < (1ll << 30), "q_temp.every");
+            }
+        need(lay_attn_fits(sp.dim, sp.vdim, true), "attention head sizes too large");
+        need(2 * sp.heads + 2 * sp.kv_heads <= 1024, "attention: too many heads");
+    } else if (type == "hgrn2") {
+        sp.mixer = LMIX_HGRN;
+        sp.heads = (int)mx->integer("heads", 0);
+        sp.kv_heads = sp.heads;
+        sp.dim = (int)mx->integer("dim", 0);
+        sp.vdim = (int)mx->integer("vdim", sp.dim);
+        need(sp.heads > 0 && sp.dim > 0 && sp.vdim > 0, "mixer sizes");
+        if (sp.dim > 256) throw CmError(CM_ERR_UNSUPPORTED, "hgrn2 head size above 256");
+    } else if (type == "parallel") {
+        const cmjson::Value* lf = mx->get("left");
+        const cmjson::Value* rg = mx->get("right");
+        need(lf && rg && lf->kind == cmjson::Value::Obj && rg->kind == cmjson::Value::Obj, "parallel layer without mixer.left / mixer.right");
+        sp.mixer = LMIX_SIDE;
+        sp.side.resize(2);
+        LayerSpec& a = sp.side[0];
+        parse_attn_sizes(*lf, a);
+        a.side_scale = (float)mx->number("left_scale", 1.0);
+        a.talk = true; a.head_norm = true;
+        if (const cmjson::Value* mk = lf->get("mask"))
+            if (mk->kind == cmjson::Value::Obj) {
+                a.win = mk->integer("size", a.win);
+                need(a.win > 0, "mask.size");
+            }
+        if (const cmjson::Value* rt = lf->get("rot"))
+            if (rt->kind == cmjson::Value::Obj) {
+                a.rot.half = true;
+                a.rot.dims = (int)rt->integer("dims", a.dim);
+                a.rot.base = rt->number("base", 10000.0);
+                need(a.rot.dims >= 0 && a.rot.dims <= a.dim && a.rot.dims % 2 == 0 && a.rot.base > 0.0, "rot.dims / rot.base");
+            }
+        need(lay_attn_talk_fits(a.heads, a.kv_heads, a.dim, a.vdim), "left mixer: head count or sizes too large");
+        need(a.heads + a.kv_heads <= 1024, "left mixer: too many heads");
+        LayerSpec& b = sp.side[1];
+        b.mixer = LMIX_SSM;
+        b.side_scale = (float)mx->number("right_scale", 1.0);
+        b.heads = (int)rg->integer("heads", 0);
+        b.kv_heads = b.heads;
+        b.vdim = (int)rg->integer("vdim", 0);
+        b.state = (int)rg->integer("state", 0);
+        b.dim = b.state;
+        b.groups = (int)rg->integer("groups", 1);
+        b.conv = (int)rg->integer("conv", 1);
+        b.norm_groups = (int)rg->integer("norm_groups", 1);
+        need(b.heads > 0 && b.vdim > 0 && b.state > 0 && b.groups > 0 && b.heads % b.groups == 0, "right mixer sizes");
+        need(b.conv >= 1 && b.conv <= 64, "right mixer: conv");
+        need(b.norm_groups > 0 && b.norm_groups <= 256 && (b.heads * b.vdim) % b.norm_groups == 0, "right mixer: norm_groups");
+        if (b.state > 256) throw CmError(CM_ERR_UNSUPPORTED, "state-space state size above 256");
+    } else throw CmError(CM_ERR_UNSUPPORTED, "layer type '" + type + "' not implemented");
+    const cmjson::Value* ml = e.get("mlp");
+    if (ml && ml->kind == cmjson::Value::Obj) {
+        need(ml->string("kind", "moe") == "moe", "mlp.kind: only 'moe'");
+        parse_mlp(ml, sp, true);
+        sp.scale_input = true; sp.expert_act = LACT_CAPGLU;
+        need(sp.limit > 0.f && (sp.shared_ff == 0 || sp.shared_limit > 0.f), "expert.limit / shared.limit");
+    }
+    if (const cmjson::Value* wo = e.get("weights_of"))
+        if (wo->kind == cmjson::Value::Num) {
+            sp.weights_of = (int)wo->num;
+            need(sp.weights_of >= 0 && sp.weights_of < (int)before.size() && before[(size_t)sp.weights_of].weights_of < 0,
+                 "weights_of names no earlier layer with tensors of its own");
+            const LayerSpec& o = before[(size_t)sp.weights_of];
+            auto same = [](const LayerSpec& x, const LayerSpec& y) {
+                return x.mixer == y.mixer && x.heads == y.heads && x.kv_heads == y.kv_heads && x.dim == y.dim && x.vdim == y.vdim && x.state == y.state &&
+                       x.groups == y.groups && x.conv == y.conv && x.rot.dims == y.rot.dims;
+            };
+            bool ok = same(sp, o) && sp.side.size() == o.side.size() && sp.mlp == o.mlp && sp.ff == o.ff && sp.experts == o.experts && sp.shared_ff == o.shared_ff;
+            for (size_t k = 0; ok && k < sp.side.size(); ++k) ok = same(sp.side[k], o.side[k]);
+            need(ok, "weights_of: the other layer's sizes differ");
+        }
+}
+
 // config.json of a layer-list decoder: "architecture", "vocab", "width", "norm".eps and "layers": [{"type", "mixer": {...}, "mlp"}]
 void Model::init_layered_config(const cmjson::Value& root) {
     const std::string arch = root.string("architecture", "");
-    if (arch != "Korupel" && arch != "Mononex" && arch != "Gibipel")
-        throw CmError(CM_ERR_UNSUPPORTED, "architecture '" + arch + "' not implemented (Korupel, Mononex, Gibipel)");
+    if (arch != "Korupel" && arch != "Mononex" && arch != "Gibipel" && arch != "Nevotar")
+        throw CmError(CM_ERR_UNSUPPORTED, "architecture '" + arch + "' not implemented (Korupel, Mononex, Gibipel, Nevotar)");
     layered = true;
     lay.reset(new Layered());
     Layered& L = *lay;
     L.parallel = arch == "Mononex";
     L.post_only = arch == "Gibipel";
-    cfg.model_type = L.parallel ? "mononex" : (L.post_only ? "gibipel" : "korupel");
+    L.pre_norm = arch == "Nevotar";
+    cfg.model_type = L.parallel ? "mononex" : (L.post_only ? "gibipel" : (L.pre_norm ? "nevotar" : "korupel"));
     if (L.post_only) {
         if (const cmjson::Value* em = root.get("embedding")) L.embed_scale = (float)em->number("scale", 1.0);
         L.logit_scale = (float)root.number("logit_scale", 1.0);
     }
     cfg.V = (int)root.integer("vocab", 0);
     cfg.H = (int)root.integer("width", 0);
-    if (const cmjson::Value* n = root.get("norm")) cfg.eps = (float)n->number("eps", 1e-6);
-    if (!L.parallel && !L.post_only) {
+    if (const cmjson::Value* n = root.get("norm")) {
+        cfg.eps = (float)n->number("eps", 1e-6);
+        if (L.pre_norm) L.norm_groups = (int)n->integer("groups", 1);
+    }
+    if (!L.parallel && !L.post_only && !L.pre_norm) {
         if (const cmjson::Value* c = root.get("canon")) L.taps = (int)c->integer("taps", 0);
         L.mult = (float)root.number("residual_mult", 1.0);
     }
     const cmjson::Value* ls = root.get("layers");
     if (!ls || ls->kind != cmjson::Value::Arr || ls->arr.empty()) throw CmError(CM_ERR_IO, "config.json: no layers");
     if (cfg.V <= 0 || cfg.H <= 0) throw CmError(CM_ERR_IO, "config.json: vocab / width missing");
+    need(L.norm_groups > 0 && L.norm_groups <= 256 && cfg.H % L.norm_groups == 0, "norm.groups");
     if (L.taps < 0 || L.taps > 64) throw CmError(CM_ERR_UNSUPPORTED, "canon.taps out of range");
     for (auto& e : ls->arr) {
         LayerSpec sp;
         if (L.parallel) parse_mononex_layer(*e, sp, L.spec);
         else if (L.post_only) parse_gibipel_layer(*e, sp);
+        else if (L.pre_norm) parse_nevotar_layer(*e, sp, L.spec);
         else parse_korupel_layer(*e, sp);
         L.spec.push_back(sp);
     }
@@ -465,11 +583,13 @@ static std::vector<float> rot_frequencies(const RotSpec& r, float* mag) {
 
 static void build_mononex(Model& m, LaySource& src);
 static void build_gibipel(Model& m, LaySource& src);
+static void build_nevotar(Model& m, LaySource& src);
 
 static void build_layered(Model& m, LaySource& src) {
     Layered& L = *m.lay;
     if (L.parallel) { build_mononex(m, src); return; }
     if (L.post_only) { build_gibipel(m, src); return; }
+    if (L.pre_norm) { build_nevotar(m, src); return; }
     const size_t W = (size_t)m.cfg.H, V = (size_t)m.cfg.V;
     const float ws = 1.0f / std::sqrt((float)W);
     m.embed = up_bf16(m, src.get("embed", V * W, 1.0f, 0.f));
@@ -732,6 +852,124 @@ static void build_gibipel(Model& m, LaySource& src) {
     m.lm_head = L.head;
 }
 
+static void build_nevotar(Model& m, LaySource& src) {
+    Layered& L = *m.lay;
+    const size_t W = (size_t)m.cfg.H, V = (size_t)m.cfg.V;
+    const float ws = 1.0f / std::sqrt((float)W);
+    m.embed = up_bf16(m, src.get("embed", V * W, 1.0f, 0.f));
+    L.w.resize(L.spec.size());
+    for (size_t i = 0; i < L.spec.size(); ++i) {
+        const LayerSpec& sp = L.spec[i];
+        if (sp.weights_of >= 0) { L.w[i] = L.w[(size_t)sp.weights_of]; continue; }      // the same tensors; its place in the pools is its own
+        LayeredLayerW& w = L.w[i];
+        const std::string p = "l" + std::to_string(i) + ".";
+        w.norm1 = up_f32(m, src.get(p + "norm1", W, 0.1f, 1.f));
+        std::vector<float> in, bias;
+        if (sp.mixer == LMIX_ATTN) {
+            // q | k | v.  The query rows are reordered so that the two maps are heads of their own whose key head follows from the usual
+            // grouping: key head (g, map m) = 2 g + m serves the query heads (2 g + m) nrep + j, j < nrep (stored: head g nrep + j, [map 1 | map 2])
+            const size_t H = (size_t)sp.heads, G = (size_t)sp.kv_heads, d = (size_t)sp.dim, e = (size_t)sp.vdim, nrep = H / G;
+            const std::string q = p + "mix.";
+            const std::vector<float> qw = src.get(q + "q", 2 * H * d * W, ws, 0.f), qb = src.get(q + "q.b", 2 * H * d, 0.1f, 0.f);
+            std::vector<float> qp(qw.size()), qbp(qb.size());
+            for (size_t h = 0; h < H; ++h)
+                for (size_t mp = 0; mp < 2; ++mp) {
+                    const size_t from = (h * 2 + mp) * d, to = ((2 * (h / nrep) + mp) * nrep + h % nrep) * d;
+                    std::copy(qw.begin() + (long)(from * W), qw.begin() + (long)((from + d) * W), qp.begin() + (long)(to * W));
+                    std::copy(qb.begin() + (long)from, qb.begin() + (long)(from + d), qbp.begin() + (long)to);
+                }
+            w.q_off = 0; w.k_off = (int)(2 * H * d); w.v_off = w.k_off + (int)(2 * G * d);
+            append(in, qp); append(bias, qbp);
+            append(in, src.get(q + "k", 2 * G * d * W, ws, 0.f)); append(bias, src.get(q + "k.b", 2 * G * d, 0.1f, 0.f));
+            append(in, src.get(q + "v", G * e * W, ws, 0.f)); append(bias, src.get(q + "v.b", G * e, 0.1f, 0.f));
+            w.in_rows = w.v_off + (int)(G * e);
+            w.g_off = w.in_rows;
+            auto dot = [&](const std::string& a, const std::string& b) {
+                const std::vector<float> x = src.get(q + a, d, 0.3f, 0.f), y = src.get(q + b, d, 0.3f, 0.f);
+                double t = 0.0;
+                for (size_t k = 0; k < d; ++k) t += (double)x[k] * (double)y[k];
+                return t;
+            };
+            w.lambda = (float)(std::exp(dot("lq1", "lk1")) - std::exp(dot("lq2", "lk2")) + (double)sp.diff);
+            w.o_w = up_bf16(m, src.get(q + "o", W * H * e, 1.0f / std::sqrt((float)(H * e)), 0.f));
+        } else if (sp.mixer == LMIX_HGRN) {
+            // q (SiLU) | forget gate (the key 1 - f takes its place) | v
+            const size_t H = (size_t)sp.heads, d = (size_t)sp.dim, e = (size_t)sp.vdim;
+            const std::string q = p + "mix.";
+            w.q_off = 0; w.k_off = (int)(H * d); w.v_off = (int)(2 * H * d); w.in_rows = (int)(2 * H * d + H * e); w.g_off = (int)(H * d);
+            append(in, src.get(q + "q", H * d * W, ws, 0.f));
+            append(in, src.get(q + "f", H * d * W, ws, 0.f));
+            append(in, src.get(q + "v", H * e * W, ws, 0.f));
+            bias.assign(H * d, 0.f);
+            append(bias, src.get(q + "f.b", H * d, 0.5f, 1.f));
+            bias.resize((size_t)w.in_rows, 0.f);
+            std::vector<float> lo = src.get(q + "lower", H * d, 0.2f, 0.4f);
+            for (float& v : lo) v = std::min(std::max(v, 0.f), 0.999f);       // a bound of a gate in (0, 1); checkpoints hold such values
+            w.lower = up_f32(m, lo);
+            w.mix_norm = up_f32(m, src.get(q + "norm", e, 0.1f, 1.f));
+            w.o_w = up_bf16(m, src.get(q + "o", W * H * e, 1.0f / std::sqrt((float)(H * e)), 0.f));
+        } else {
+            w.side.resize(2);
+            const LayerSpec &sa = sp.side[0], &sb = sp.side[1];
+            LayeredLayerW &wa = w.side[0], &wb = w.side[1];
+            {   // left: q | k | v, biases on all three
+                const size_t H = (size_t)sa.heads, G = (size_t)sa.kv_heads, d = (size_t)sa.dim, e = (size_t)sa.vdim;
+                const std::string q = p + "mix.left.";
+                wa.q_off = 0; wa.k_off = (int)(H * d); wa.v_off = wa.k_off + (int)(G * d);
+                append(in, src.get(q + "q", H * d * W, ws, 0.f)); append(bias, src.get(q + "q.b", H * d, 0.1f, 0.f));
+                append(in, src.get(q + "k", G * d * W, ws, 0.f)); append(bias, src.get(q + "k.b", G * d, 0.1f, 0.f));
+                append(in, src.get(q + "v", G * e * W, ws, 0.f)); append(bias, src.get(q + "v.b", G * e, 0.1f, 0.f));
+                wa.q_norm = up_f32(m, src.get(q + "q.norm", d, 0.1f, 1.f));
+                wa.k_norm = up_f32(m, src.get(q + "k.norm", d, 0.1f, 1.f));
+                wa.talk = up_f32(m, src.get(q + "talk", H * H, 0.6f / std::sqrt((float)H), 0.f));
+                if (sa.rot.dims > 0) wa.rot_freq = up_f32(m, rot_frequencies(sa.rot, &wa.rot_mag));
+                wa.o_col = 0;
+            }
+            {   // right: z | x | B | C | dt
+                const size_t H = (size_t)sb.heads, e = (size_t)sb.vdim, N = (size_t)sb.state, Gr = (size_t)sb.groups, inner = H * e;
+                const size_t C = inner + 2 * Gr * N, taps = (size_t)sb.conv;
+                const std::string q = p + "mix.right.";
+                const int base = (int)(in.size() / W);
+                wb.z_off = base; wb.x_off = base + (int)inner; wb.dt_off = wb.x_off + (int)C;
+                wb.v_off = 0; wb.k_off = (int)inner; wb.q_off = (int)(inner + Gr * N);       // inside the convolved channels: x | B | C
+                append(in, src.get(q + "in", (2 * inner + 2 * Gr * N + H) * W, ws, 0.f));
+                wb.conv_w = up_f32(m, src.get(q + "conv", C * taps, 0.5f / std::sqrt((float)taps), 0.f));
+                wb.conv_b = up_f32(m, src.get(q + "conv.b", C, 0.1f, 0.f));
+                wb.dt_bias = up_f32(m, src.get(q + "dt_bias", H, 0.5f, -1.f));
+                std::vector<float> an = src.get(q + "A_log", H, 0.5f, 0.f);
+                for (float& v : an) v = (float)(-std::exp((double)v));
+                wb.a_neg = up_f32(m, an);
+                wb.skip = up_f32(m, src.get(q + "D", H, 0.3f, 1.f));
+                wb.mix_norm = up_f32(m, src.get(q + "norm", inner, 0.1f, 1.f));
+                wb.o_col = sa.heads * sa.vdim;
+            }
+            w.in_rows = (int)(in.size() / W);
+            w.g_off = w.in_rows;
+            bias.resize((size_t)w.in_rows, 0.f);
+            {   // one output projection for both mixers: the input columns are [left heads | right heads]
+                const size_t ka = (size_t)sa.heads * sa.vdim, kb = (size_t)sb.heads * sb.vdim, K = ka + kb;
+                const std::vector<float> oa = src.get(p + "mix.left.o", W * ka, 1.0f / std::sqrt((float)ka), 0.f);
+                const std::vector<float> ob = src.get(p + "mix.right.o", W * kb, 1.0f / std::sqrt((float)kb), 0.f);
+                std::vector<float> o(W * K);
+                for (size_t r = 0; r < W; ++r) {
+                    std::copy(oa.begin() + (long)(r * ka), oa.begin() + (long)((r + 1) * ka), o.begin() + (long)(r * K));
+                    std::copy(ob.begin() + (long)(r * kb), ob.begin() + (long)((r + 1) * kb), o.begin() + (long)(r * K + ka));
+                }
+                w.o_w = up_bf16(m, o);
+            }
+        }
+        w.in_w = up_bf16(m, in);
+        w.in_b = up_f32(m, bias);
+        if (sp.mlp == LMLP_MOE) {
+            w.norm2 = up_f32(m, src.get(p + "norm2", W, 0.1f, 1.f));
+            build_experts(m, src, p, sp, w);
+        }
+    }
+    L.final_norm = up_f32(m, src.get("final.norm", W, 0.1f, 1.f));
+    L.head = m.embed;                      // the logits come from the embedding table
+    m.lm_head = L.head;
+}
+
 void load_layered_from_dir(Model& m, const std::string& dir) {
     try {
         LayFileSource src(dir);
@@ -772,7 +1010,7 @@ void Model::alloc_runtime_layered() {
             } else {
                 if (kv_index[i] < 0) kv_index[i] = n_kv_layers++;
                 w.kv_idx = kv_index[i];
-                w.k_page_bytes = (size_t)sp.kv_heads * page * dk * kv_esize;
+                w.k_page_bytes = (size_t)sp.kv_heads * sp.maps * page * dk * kv_esize;      // every map of a key head has rows of its own
                 w.k_pool_off = pool_bytes;
                 pool_bytes += (size_t)n_pages * w.k_page_bytes;
                 page_bytes += w.k_page_bytes;      // all layers' share of one page (kv_bytes)
@@ -802,7 +1040,7 @@ void Model::alloc_runtime_layered() {
             }
             const int nrep = sp.heads / sp.kv_heads;
             if (std::find(L.nreps.begin(), L.nreps.end(), nrep) == L.nreps.end()) L.nreps.push_back(nrep);
-            L.max_o = std::max(L.max_o, sp.heads * ev);
+            L.max_o = std::max(L.max_o, sp.heads * sp.maps * ev);
             L.max_e = std::max(L.max_e, ev);
             if (sp.mixer == LMIX_LATENT) {
                 L.max_o = std::max(L.max_o, sp.heads * sp.vdim);
@@ -817,11 +1055,22 @@ void Model::alloc_runtime_layered() {
             L.max_o = std::max(L.max_o, sp.heads * (sp.vdim + 1));
             L.max_ld = std::max(L.max_ld, sp.heads);
             L.max_mh = std::max(L.max_mh, sp.heads);
+        } else if (sp.mixer == LMIX_SSM) {
+            // state [H][N][e]; the convolution's last taps - 1 inputs [taps - 1][x | B | C]
+            w.st_off = st;
+            st += (size_t)sp.heads * sp.state * sp.vdim;
+            const int C = sp.heads * sp.vdim + 2 * sp.groups * sp.state;
+            w.cv_off = cv;
+            cv += (size_t)(sp.conv - 1) * C;
+            L.max_conv = std::max(L.max_conv, C);
+            L.max_o = std::max(L.max_o, sp.heads * sp.vdim);
+            L.max_ld = std::max(L.max_ld, sp.heads);
+            L.max_mh = std::max(L.max_mh, sp.heads);
         } else {
             w.st_off = st;
             st += (size_t)sp.heads * sp.dim * sp.vdim;
             L.max_o = std::max(L.max_o, sp.heads * sp.vdim);
-            if (sp.mixer == LMIX_GLA) L.max_ld = std::max(L.max_ld, sp.heads * sp.dim);
+            if (sp.mixer == LMIX_GLA || sp.mixer == LMIX_HGRN) L.max_ld = std::max(L.max_ld, sp.heads * sp.dim);
         }
     };
     for (size_t i = 0; i < L.spec.size(); ++i) {
@@ -882,6 +1131,7 @@ void Model::alloc_runtime_layered() {
     if (L.max_ld) L.LD = dalloc<float>(cap * (size_t)L.max_ld);
     if (L.max_mh) { L.KM = dalloc<float>(cap * (size_t)L.max_mh); L.MR = dalloc<float>(cap * (size_t)L.max_mh); }
     if (L.max_sff) L.HS = dalloc<float>(cap * (size_t)L.max_sff);
+    if (L.max_conv) L.XB = dalloc<float>(cap * (size_t)L.max_conv);
     if (L.max_E > 1 || L.max_top > 1 || std::any_of(L.spec.begin(), L.spec.end(), [](const LayerSpec& s) { return s.mlp == LMLP_MOE; })) {
         L.YS = dalloc<float>(cap * (size_t)L.max_slots * W);
         L.wsel = dalloc<float>(cap * (size_t)L.max_slots);
@@ -901,8 +1151,9 @@ void Model::alloc_runtime_layered() {
     }
     size_t hde = 0, hd = 0;
     auto chunk_scratch = [&](const LayerSpec& sp) {
-        if ((sp.mixer == LMIX_LIGHTNING || sp.mixer == LMIX_GLA) && sp.dim <= 128) hde = std::max(hde, (size_t)sp.heads * sp.dim * sp.vdim);
-        if (sp.mixer == LMIX_GLA && sp.dim <= 128) hd = std::max(hd, (size_t)sp.heads * sp.dim);
+        const bool lin = sp.mixer == LMIX_LIGHTNING || sp.mixer == LMIX_GLA || sp.mixer == LMIX_HGRN || sp.mixer == LMIX_SSM;
+        if (lin && sp.dim <= 128) hde = std::max(hde, (size_t)sp.heads * sp.dim * sp.vdim);
+        if (lin && sp.mixer != LMIX_LIGHTNING && sp.dim <= 128) hd = std::max(hd, (size_t)sp.heads * sp.dim);
         if (sp.mixer == LMIX_MEMORY && sp.dim <= 128) {
             hde = std::max(hde, (size_t)sp.heads * sp.dim * (sp.vdim + 1));
             hd = std::max(hd, (size_t)sp.heads * sp.dim);
@@ -1128,8 +1379,9 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
         };
         // softmax attention of one layer over the pages: queries at qsrc[row ldq + q_off + head dk], output [T][H ev] into L.O
         auto run_attention = [&](const LayerSpec& sp, const LayeredLayerW& w, const float* qsrc, int ldq, int q_off, int g_off, int dk, int ev,
-                                 float* out = nullptr, int ldo = 0, float out_scale = 1.f) {
+                                 float* out = nullptr, int ldo = 0, float out_scale = 1.f, int v_div = 1) {
             LAttnArgs a;
+            a.v_div = v_div;
             a.proj = qsrc; a.ldp = ldq; a.q_off = q_off; a.g_off = g_off;
             a.out = out ? out : L.O; a.ldo = out ? ldo : sp.heads * ev; a.out_scale = out_scale;
             if (sp.pool > 0) {
@@ -1178,6 +1430,19 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                 a.U = L.U; a.chunks = (const int2*)(L.d_tab + o_chunks); a.nchunks = nchunks;
             }
             launch_lay_lightning(a, s);
+        };
+        // long portions in the pass: the linear-attention kernels run parallel over chunks
+        auto linear_chunks = [&](LLightArgs& a) {
+            if (L.U && max_n > LAY_LIGHT_CHUNK && a.d <= 128) {
+                a.U = L.U; a.chunks = (const int2*)(L.d_tab + o_chunks); a.nchunks = nchunks;
+                if (a.ldec) a.D = L.Dch;
+            }
+        };
+        // pre-norm layers: the finished sublayer's rows (nsum per token, summed in order) join the residual inside the next norm's launch
+        struct { const float* y = nullptr; int nsum = 1; } padd;
+        auto add_gnorm = [&](const float* nw_, float* out) {
+            launch_lay_add_gnorm(L.X, nullptr, padd.y, padd.nsum, nw_, out, T, W, L.norm_groups, cfg.eps, s);
+            padd.y = nullptr;
         };
         const float *par_y1 = nullptr, *par_y2 = nullptr;       // parallel layers: sublayer outputs not yet added to the residual
         for (size_t li = 0; li < L.spec.size(); ++li) {
@@ -1262,6 +1527,122 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                     launch_lay_add_rows(L.X, par_y1, par_y2, (size_t)T * W, s);
                     par_y1 = par_y2 = nullptr;
                 }
+            } else if (L.pre_norm) {
+                // ---- x += mixer(norm1 x), x += ff(norm2 x), norms in equal parts
+                add_gnorm(w.norm1, L.Hc);
+                LGemmArgs g;
+                g.A = L.Hc; g.lda = W; g.W = w.in_w; g.bias = w.in_b; g.C = L.P; g.ldc = w.in_rows; g.M = T; g.N = w.in_rows; g.K = W;
+                g.act_split = w.g_off; g.act = sp.mixer == LMIX_HGRN ? LACT_SILU : LACT_NONE; g.act2 = LACT_NONE;
+                lay_gemm(*this, L, g, 1, s);
+                const float* oa = L.O;
+                int on = 0;
+                if (sp.mixer == LMIX_ATTN) {
+                    // two maps per head as heads of their own (2 H query heads over 2 G key heads, pairs of key heads share a value head)
+                    const int H = sp.heads, G = sp.kv_heads, d = sp.dim, e = sp.vdim;
+                    LQkPrepExtra ex;
+                    ex.Gv = G; ex.qt_coef = sp.qt_coef; ex.qt_every = (int)sp.qt_every;
+                    launch_lay_qk_prep(L.P, w.in_rows, w.q_off, w.k_off, w.v_off, 2 * H, 2 * G, d, e, nullptr, nullptr, cfg.eps, 0, false, nullptr, 1.f,
+                                       kv_pool + w.k_pool_off, kv_pool + w.v_pool_off, kv_mode, d_bt, d_segs, d_rowseg, T, page, s, 0, 0, nullptr, nullptr, &ex);
+                    LayerSpec two = sp;
+                    two.heads = 2 * H; two.kv_heads = 2 * G;
+                    run_attention(two, w, L.P, w.in_rows, w.q_off, 0, d, e, nullptr, 0, 1.f, 2);
+                    launch_lay_diff_combine(L.O, L.O2, T, H, G, e, w.lambda, 1.f - sp.diff, cfg.eps, s);
+                    oa = L.O2; on = H * e;
+                } else if (sp.mixer == LMIX_HGRN) {
+                    const int H = sp.heads, d = sp.dim, e = sp.vdim;
+                    launch_lay_hgrn_gates(L.P, w.in_rows, w.k_off, w.lower, L.LD, T, H * d, s);
+                    LLightArgs a;
+                    a.proj = L.P; a.ldp = w.in_rows; a.q_off = w.q_off; a.k_off = w.k_off; a.v_off = w.v_off;
+                    a.out = L.O; a.ldo = H * e;
+                    a.state_pool = state_pool; a.slot_stride = state_slot_elems; a.st_off = w.st_off;
+                    a.segs = d_segs; a.nseg = nseg; a.decay = nullptr; a.H = H; a.d = d; a.e = e; a.all_single = all_decode;
+                    a.ldec = L.LD; a.ldd = H * d;
+                    linear_chunks(a);
+                    launch_lay_lightning(a, s);
+                    launch_lay_rms_gate(L.O, nullptr, 0, w.mix_norm, L.O2, T, H * e, cfg.eps, s, e, true);
+                    oa = L.O2; on = H * e;
+                } else {
+                    for (const LayerSpec& sd : sp.side) on += sd.heads * sd.vdim;
+                    for (size_t k = 0; k < sp.side.size(); ++k) {
+                        const LayerSpec& sd = sp.side[k];
+                        const LayeredLayerW& sw = w.side[k];
+                        const int H = sd.heads, e = sd.vdim;
+                        if (sd.mixer == LMIX_ATTN) {
+                            const int G = sd.kv_heads, d = sd.dim;
+                            LQkPrepExtra ex;
+                            ex.head_norm = sd.head_norm;
+                            launch_lay_qk_prep(L.P, w.in_rows, sw.q_off, sw.k_off, sw.v_off, H, G, d, e, sw.q_norm, sw.k_norm, cfg.eps, sd.rot.dims,
+                                               sd.rot.half, sd.rot.dims > 0 ? sw.rot_freq : nullptr, sw.rot_mag, kv_pool + sw.k_pool_off,
+                                               kv_pool + sw.v_pool_off, kv_mode, d_bt, d_segs, d_rowseg, T, page, s, 0, 0, nullptr, nullptr, &ex);
+                            LAttnArgs a;
+                            a.proj = L.P; a.ldp = w.in_rows; a.q_off = sw.q_off; a.g_off = 0;
+                            a.out = L.O + sw.o_col; a.ldo = on; a.out_scale = sd.side_scale;
+                            a.kpool = kv_pool + sw.k_pool_off; a.vpool = kv_pool + sw.v_pool_off; a.bt = d_bt; a.segs = d_segs;
+                            a.tiles = nullptr; a.ntiles = 0; a.r1 = a.r2 = nullptr;
+                            a.H = H; a.G = G; a.d = d; a.e = e; a.page = page; a.scale = sd.scale; a.win = sd.win; a.keep = 0;
+                            a.bias = LBIAS_NONE; a.gate = LGATE_NONE;
+                            if (all_decode) {      // few rows, many keys: the window's key tiles are dealt to several blocks
+                                const long long seen = std::min<long long>(max_len, sd.win);
+                                const int key_tiles = (int)((seen + 31) / 32);
+                                a.nsplit = std::max(1, std::min({32, key_tiles, 256 / std::max(1, nseg), Layered::ATT_PARTS * 16 / std::max(1, nseg * H)}));
+                                a.part_o = L.att_po; a.part_ml = L.att_pml;
+                            }
+                            launch_lay_attn_talk(a, sw.talk, nseg, max_n, kv_mode, s);
+                        } else if (sd.mixer == LMIX_SSM) {
+                            const int N = sd.state, C = H * e + 2 * sd.groups * N;
+                            LConvArgs c;
+                            c.src = L.P; c.lds = w.in_rows; c.off = sw.x_off; c.C = C; c.dst = L.XB; c.ldd = C; c.cw = sw.conv_w; c.cb = sw.conv_b;
+                            c.taps = sd.conv; c.act = LACT_SILU; c.conv_pool = conv_pool; c.slot_stride = conv_slot_elems; c.cv_off = sw.cv_off;
+                            c.segs = d_segs; c.rowseg = d_rowseg;
+                            c.H = H; c.dt_off = sw.dt_off; c.dt_bias = sw.dt_bias; c.a_neg = sw.a_neg; c.ldec = L.LD; c.kmul = L.KM;
+                            c.tail_too = all_decode;
+                            launch_lay_conv_act(c, T, s);
+                            if (!all_decode) launch_lay_conv_tail(c, nseg, s);
+                            LLightArgs a;
+                            a.proj = L.XB; a.ldp = C; a.q_off = sw.q_off; a.k_off = sw.k_off; a.v_off = sw.v_off;
+                            a.out = L.O2; a.ldo = H * e;
+                            a.state_pool = state_pool; a.slot_stride = state_slot_elems; a.st_off = sw.st_off;
+                            a.segs = d_segs; a.nseg = nseg; a.decay = nullptr; a.H = H; a.d = N; a.e = e; a.all_single = all_decode;
+                            a.ldec = L.LD; a.ldd = H; a.head_decay = true; a.kmul = L.KM; a.qk_rep = H / sd.groups;
+                            linear_chunks(a);
+                            launch_lay_lightning(a, s);
+                            launch_lay_ssm_out(L.O2, L.XB, C, 0, L.P, w.in_rows, sw.z_off, sw.skip, sw.mix_norm, L.O + sw.o_col, on, T, H, e,
+                                               sd.norm_groups, cfg.eps, sd.side_scale, s);
+                        } else throw CmError(CM_ERR_UNSUPPORTED, "side mixer kind");
+                    }
+                }
+                LGemmArgs go;
+                go.A = oa; go.lda = on; go.W = w.o_w; go.C = L.Y; go.ldc = W; go.M = T; go.N = W; go.K = on;
+                lay_gemm(*this, L, go, 1, s);
+                padd.y = L.Y; padd.nsum = 1;
+                if (sp.mlp == LMLP_MOE) {
+                    add_gnorm(w.norm2, L.Hc);
+                    // an expert's weight multiplies its INPUT: the rows of the grouped product are w h, and the combine is a plain sum
+                    const int slots = sp.top + (sp.shared_ff > 0 ? 1 : 0);
+                    launch_lay_router(L.Hc, w.router, L.sel, L.wsel, T, W, sp.experts, sp.top, s, &sp.router, nullptr, slots, L.Z);
+                    launch_lay_moe_plan(L.sel, L.off, L.srt, T * sp.top, sp.experts, s, sp.top, slots);
+                    LGemmArgs gu;
+                    gu.A = L.Hc; gu.lda = W; gu.a_idx = L.srt; gu.a_div = slots; gu.a_scale = sp.scale_input ? L.wsel : nullptr;
+                    gu.W = w.gate; gu.W2 = w.up; gu.w_stride = (size_t)sp.ff * W;
+                    gu.C = L.HH; gu.ldc = sp.ff; gu.M = T; gu.N = sp.ff; gu.K = W; gu.grp_off = L.off; gu.act = sp.expert_act; gu.act_param = sp.limit;
+                    lay_gemm(*this, L, gu, sp.experts, s);
+                    LGemmArgs dn;
+                    dn.A = L.HH; dn.lda = sp.ff; dn.W = w.down; dn.w_stride = (size_t)W * sp.ff;
+                    dn.C = L.YS; dn.ldc = W; dn.c_idx = L.srt; dn.M = T; dn.N = W; dn.K = sp.ff; dn.grp_off = L.off;
+                    lay_gemm(*this, L, dn, sp.experts, s);
+                    if (sp.shared_ff > 0) {        // the expert every token uses: row `top` of the token's rows
+                        LGemmArgs su;
+                        su.A = L.Hc; su.lda = W; su.W = w.sh_gate; su.W2 = w.sh_up; su.C = L.HS; su.ldc = sp.shared_ff; su.M = T; su.N = sp.shared_ff;
+                        su.K = W; su.act = sp.expert_act; su.act_param = sp.shared_limit;
+                        lay_gemm(*this, L, su, 1, s);
+                        LGemmArgs sdn;
+                        sdn.A = L.HS; sdn.lda = sp.shared_ff; sdn.W = w.sh_down; sdn.C = L.YS + (size_t)sp.top * W; sdn.ldc = slots * W; sdn.M = T;
+                        sdn.N = W; sdn.K = sp.shared_ff;
+                        lay_gemm(*this, L, sdn, 1, s);
+                    }
+                    padd.y = L.YS; padd.nsum = slots;
+                }
+                if (L.capture || li + 1 == L.spec.size()) add_gnorm(nullptr, nullptr);
             } else if (L.post_only) {
                 // ---- the sublayers read the residual itself; x += g * unit(sublayer(x)).  All mixers of the layer share one input
                 // projection and one output projection (their heads side by side in its input, each times its scale)
@@ -1411,7 +1792,8 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
         // ---- final norm + head over the wanted rows, LOGIT_ROWS at a time
         for (int w0 = 0; w0 < nw; w0 += Layered::LOGIT_ROWS) {
             const int nr = std::min(Layered::LOGIT_ROWS, nw - w0);
-            launch_lay_rms_rows(L.X, d_wrows + w0, L.final_norm, L.Xw, nr, W, cfg.eps, s);
+            if (L.pre_norm) launch_lay_add_gnorm(L.X, d_wrows + w0, nullptr, 0, L.final_norm, L.Xw, nr, W, L.norm_groups, cfg.eps, s);
+            else launch_lay_rms_rows(L.X, d_wrows + w0, L.final_norm, L.Xw, nr, W, cfg.eps, s);
             LGemmArgs hd;
             hd.A = L.Xw; hd.lda = W; hd.W = L.head; hd.C = logitsb; hd.ldc = V; hd.M = nr; hd.N = V; hd.K = W;
             lay_gemm(*this, L, hd, 1, s);
