@@ -146,7 +146,7 @@ def relaunch_under_torchrun(n: int) -> int:
 
 
 def korupel_leg(args, names=None, prompt_lens=None, label="korupel"):
-    """--korupel / --mononex / --gibipel: prompt and decode throughput of a layer-list decoder (Korupel, Mononex, Gibipel; crane_amd/csrc/model_layered.cpp)
+    """--korupel / --mononex / --gibipel / --nevotar: prompt and decode throughput of a layer-list decoder (Korupel, Mononex, Gibipel, Nevotar; crane_amd/csrc/model_layered.cpp)
     at the widths of a real model, random weights, beside the closest family of the library at equal size: the Qwen3.5 hybrid
     (linear attention 3 : 1 softmax attention, same width / ff / layers / vocabulary).  One JSON line; the default workload of this
     script is not touched."""
@@ -253,6 +253,9 @@ def main():
     ap.add_argument("--gibipel", default=None, metavar="CONFIGS", help="comma-separated registry configs (e.g. "
                     "gibipel-1b,korupel-1b-moe,qwen3.5-0.8b): prompt and decode throughput of each instead of the headline workload")
     ap.add_argument("--gibipel-prompts", default="512,2048", help="prompt lengths of --gibipel")
+    ap.add_argument("--nevotar", default=None, metavar="CONFIGS", help="comma-separated registry configs (e.g. "
+                    "nevotar-1b,gibipel-1b,korupel-1b-moe): prompt and decode throughput of each instead of the headline workload")
+    ap.add_argument("--nevotar-prompts", default="512,2048", help="prompt lengths of --nevotar")
     args = ap.parse_args()
     if args.korupel:
         sys.exit(korupel_leg(args))
@@ -260,6 +263,8 @@ def main():
         sys.exit(korupel_leg(args, args.mononex, args.mononex_prompts, "mononex"))
     if args.gibipel:
         sys.exit(korupel_leg(args, args.gibipel, args.gibipel_prompts, "gibipel"))
+    if args.nevotar:
+        sys.exit(korupel_leg(args, args.nevotar, args.nevotar_prompts, "nevotar"))
 
     if args.tp_inprocess:      # ranks that share a device need one hardware queue per rank stream: before the HIP runtime starts
         os.environ.setdefault("GPU_MAX_HW_QUEUES", "16")

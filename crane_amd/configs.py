@@ -270,6 +270,54 @@ CONFIGS.update({
 })
 
 
+# ---- layer-list decoders: Nevotar ------------------------------------------------------------------------------------------
+def nevotar_config(vocab: int, width: int, kinds: "list | tuple", heads: int, kv_heads: int, dim: int, vdim: int, window: int,
+                   rec_heads: int, rec_dim: int, rec_vdim: int, ssm_heads: int, ssm_vdim: int, state: int, ssm_groups: int, experts: int,
+                   top: int, expert_ff: int, shared_ff: int = 0, limit: float = 7.0, diff: float = 0.6, q_coef: float = 0.1, q_every: int = 1024,
+                   rot_dims: "int | None" = None, rot_base: float = 1000000.0, conv: int = 4, ssm_norm_groups: int = 1, left_scale: float = 1.0,
+                   right_scale: float = 1.0, norm_groups: int = 1, eps: float = 1e-6, no_ff: "tuple | list" = (), weights_of: "dict | None" = None) -> dict:
+    """Pre-norm layers of the kinds named in `kinds`: "attention" (two softmax maps per head, `dim` per map), "hgrn2" (gated
+    recurrence) and "parallel" (window attention with mixed heads beside a state-space mixer); mixture-of-experts feed-forwards
+    (layers in `no_ff`: none); weights_of[i] = j lets layer i run on layer j's tensors."""
+    made = []
+    for i, kind in enumerate(kinds):
+        if kind == "attention":
+            mx = dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, diff=diff, q_temp=dict(coef=q_coef, every=q_every), scale=dim ** -0.5)
+        elif kind == "hgrn2":
+            mx = dict(heads=rec_heads, dim=rec_dim, vdim=rec_vdim)
+        else:
+            mx = dict(left=dict(heads=heads, kv_heads=kv_heads, dim=dim, vdim=vdim, scale=dim ** -0.5, mask=dict(size=window),
+                                rot=dict(base=rot_base, dims=dim if rot_dims is None else rot_dims)),
+                      right=dict(heads=ssm_heads, vdim=ssm_vdim, state=state, groups=ssm_groups, conv=conv, norm_groups=ssm_norm_groups),
+                      left_scale=left_scale, right_scale=right_scale)
+        mlp = None
+        if i not in no_ff:
+            mlp = dict(kind="moe", expert=dict(ff=expert_ff, limit=limit), router=dict(experts=experts, top=top))
+            if shared_ff:
+                mlp["shared"] = dict(ff=shared_ff, limit=limit)
+        ly = dict(type=kind, mixer=mx, mlp=mlp)
+        if weights_of and i in weights_of:
+            ly = dict(copy.deepcopy(made[weights_of[i]]), weights_of=weights_of[i])
+        made.append(ly)
+    return dict(architecture="Nevotar", vocab=vocab, width=width, norm=dict(eps=eps, groups=norm_groups), layers=made)
+
+
+_NEVOTAR_1B = dict(heads=8, kv_heads=2, dim=128, vdim=128, window=1024, rec_heads=8, rec_dim=128, rec_vdim=128, ssm_heads=16, ssm_vdim=64,
+                   state=128, ssm_groups=2, experts=14, top=4, expert_ff=768, shared_ff=512, rot_dims=64, ssm_norm_groups=2, norm_groups=2)
+CONFIGS.update({
+    "tiny-nevotar": nevotar_config(320, 128, ["attention", "hgrn2", "parallel", "parallel", "attention"], heads=4, kv_heads=2, dim=16, vdim=24,
+                                   window=20, rec_heads=2, rec_dim=16, rec_vdim=24, ssm_heads=4, ssm_vdim=8, state=16, ssm_groups=2, experts=6,
+                                   top=2, expert_ff=48, shared_ff=64, limit=1.5, q_every=16, rot_dims=8, ssm_norm_groups=2, left_scale=0.7,
+                                   right_scale=1.2, norm_groups=4, no_ff=(1,), weights_of={3: 2, 4: 0}),
+    # the widths of korupel-1b-moe / gibipel-1b (1024 wide, 24 layers, vocabulary 248 320, 8 query / 2 key heads of 128): 6 layers of
+    # two-map attention over the whole context, 6 gated recurrences of 8 heads of 128 x 128, 12 layers of window attention (1024, mixed
+    # heads, half of a head rotates) beside a state-space mixer of 16 heads of 128 x 64; 14 experts of 768, 4 per token, and a shared
+    # expert of 512 (3584 active inner columns, as the dense models)
+    "nevotar-1b": nevotar_config(248320, 1024, ["attention", "hgrn2", "parallel", "parallel"] * 6, **_NEVOTAR_1B),
+    "nevotar-1b-4l": nevotar_config(32768, 1024, ["attention", "hgrn2", "parallel", "parallel"], **_NEVOTAR_1B),
+})
+
+
 def get_config(name: str) -> dict:
     if name not in CONFIGS:
         raise KeyError(f"unknown config {name!r}; have {sorted(CONFIGS)}")

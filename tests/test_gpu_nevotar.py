@@ -1,0 +1,548 @@
+"""GPU: the Nevotar decoder in the library (kernels_layered.hip, kernels_layered_mix.hip, model_layered.cpp, the engine's mixed
+steps) against the plain NumPy statement oracle/nevotar_oracle.py, on small configurations with random weights made here.
+
+float32 compute is the sharp comparison (TOL_F32 relative to the largest logit); bfloat16 compute is checked against the
+same oracle with the rounding's own allowance, and against itself across schedules."""
+import numpy as np
+import pytest
+
+from oracle import nevotar_oracle as O
+from tests import nevotar_util as U
+
+pytestmark = pytest.mark.gpu
+
+TOL_F32 = 2e-4
+TOL_BF16 = 6e-2
+
+
+def _load(tmp_path, cfg, P, dtype="float32", **kw):
+    from crane_amd.backend import Model
+    kw.setdefault("max_seq_len", 512)
+    kw.setdefault("max_seqs", 4)
+    return Model.from_pretrained(U.write_checkpoint(str(tmp_path / "ckpt"), cfg, P), compute_dtype=dtype, **kw)
+
+
+def _err(got, want):
+    want = np.asarray(want, np.float64)
+    return float(np.abs(np.asarray(got, np.float64) - want).max() / np.abs(want).max())
+
+
+def _err_most(got, want, median=0.015):
+    """bfloat16 format: the error that nine positions in ten stay under.  A router's close call that the rounding decides the other
+    way moves one position by a whole expert (and, through the recurrent mixers, a few after it a little); no test rests on those."""
+    want = np.asarray(want, np.float64)
+    per = np.abs(np.asarray(got, np.float64) - want).max(-1) / np.abs(want).max()
+    assert np.median(per) < median, float(np.median(per))
+    return float(np.quantile(per, 0.9))
+
+
+def _err_long(got, want):
+    """bfloat16 format over hundreds of positions and three routed layers: the few router calls that fall the other way travel on
+    through the recurrent states and the causal attention, so the bounds are wider; the float32 run of the same test is the sharp one."""
+    return _err_most(got, want, 0.06) / 2.5
+
+
+def _all(n):
+    return list(range(n))
+
+
+def _par(lf, rg, mlp=None, ls=0.8, rs=1.1):
+    return U.layer("parallel", U.side(lf, rg, ls, rs), mlp)
+
+
+SINGLE = {
+    "differential attention alone": U.config([U.layer("attention", U.attn(), None)]),
+    "differential attention, every head its own keys, one norm part, no query growth": U.config(
+        [U.layer("attention", U.attn(heads=3, kv_heads=3, dim=20, vdim=12, diff=0.2, coef=0.0, every=1), None)], groups=1),
+    "differential attention, one key head, the query grows at every position": U.config(
+        [U.layer("attention", U.attn(heads=5, kv_heads=1, dim=8, vdim=24, diff=0.8, coef=0.6, every=1, scale=0.5), None)], groups=2),
+    "gated recurrence alone": U.config([U.layer("hgrn2", U.hgrn(), None)]),
+    "gated recurrence, one head": U.config([U.layer("hgrn2", U.hgrn(heads=1, dim=20, vdim=7), None)], groups=6),
+    "window attention with mixed heads alone": U.config([_par(U.left(), U.right(), None, 1.0, 0.0)]),
+    "window attention, every head its own keys, nothing rotates": U.config([_par(U.left(heads=3, kv_heads=3, dim=12, vdim=20, size=11, dims=0), U.right(), None, 1.0, 0.0)]),
+    "window attention, a quarter of a head rotates, five heads": U.config([_par(U.left(heads=5, kv_heads=1, dim=24, vdim=6, size=14, dims=6, base=50.0), U.right(), None, 1.0, 0.0)]),
+    "state-space mixer alone": U.config([_par(U.left(), U.right(), None, 0.0, 1.0)]),
+    "state-space mixer, one group, one norm part, two taps": U.config([_par(U.left(), U.right(heads=3, vdim=10, state=6, groups=1, conv=2, norm_groups=1), None, 0.0, 1.0)]),
+    "state-space mixer, every head its own group, one tap": U.config([_par(U.left(), U.right(heads=2, vdim=8, state=20, groups=2, conv=1, norm_groups=4), None, 0.0, 1.0)]),
+    "both mixers side by side": U.config([_par(U.left(), U.right(), None, 0.7, 1.2)]),
+    "experts with a shared expert, two per token": U.config([U.layer("hgrn2", U.hgrn(), U.moe(experts=6, top=2, ff=24, limit=0.6, shared=40, shared_limit=2.0))]),
+    "experts without a shared expert, one per token": U.config([U.layer("hgrn2", U.hgrn(), U.moe(experts=3, top=1, ff=20, limit=1.0, shared=0))]),
+    "every expert chosen": U.config([U.layer("hgrn2", U.hgrn(), U.moe(experts=4, top=4, ff=12, limit=3.0, shared=8))]),
+}
+
+
+@pytest.mark.parametrize("name", list(SINGLE))
+def test_each_mechanism_alone_whole_prompt_and_layer_rows(tmp_path, name):
+    cfg = SINGLE[name]
+    P = U.random_weights(cfg, 1)
+    toks = U.tokens(41, cfg["vocab"], 1)
+    want, layers = O.forward(cfg, P, toks, True)
+    m = _load(tmp_path, cfg, P)
+    try:
+        m.layer_capture(True)
+        s = m.seq_alloc()
+        got, greedy = m.step_batch([(s, toks, _all(len(toks)))])
+        rows = m.layer_rows().reshape(len(cfg["layers"]), len(toks), cfg["width"])
+        assert _err(rows, layers) < TOL_F32
+        assert _err(got, want) < TOL_F32
+        assert list(greedy) == [int(np.argmax(r)) for r in got]
+    finally:
+        m.close()
+
+
+def test_prefill_against_token_by_token_decoding(tmp_path):
+    cfg = U.small_config()
+    P = U.random_weights(cfg, 2)
+    toks = U.tokens(70, cfg["vocab"], 2)
+    want = O.forward(cfg, P, toks)
+    m = _load(tmp_path, cfg, P)
+    try:
+        a, b = m.seq_alloc(), m.seq_alloc()
+        whole, _ = m.step_batch([(a, toks, _all(len(toks)))])
+        serial = np.concatenate([m.step_batch([(b, [t], [0])])[0] for t in toks])
+        assert _err(whole, want) < TOL_F32 and _err(serial, want) < TOL_F32
+        assert _err(serial, whole) < TOL_F32
+    finally:
+        m.close()
+
+
+@pytest.mark.parametrize("cuts", [[2] * 12 + [3, 5, 2, 7, 1, 1, 2, 16, 2], [64, 2, 1, 3], [1, 69], [33, 33, 4], [5, 60, 2, 2, 1]])
+def test_portions_of_several_sizes_down_to_two_tokens(tmp_path, cuts):
+    cfg = U.small_config()
+    P = U.random_weights(cfg, 3)
+    n = sum(cuts)
+    toks = U.tokens(n, cfg["vocab"], 3)
+    want = O.forward(cfg, P, toks)
+    m = _load(tmp_path, cfg, P)
+    try:
+        s, at, out = m.seq_alloc(), 0, []
+        for c in cuts:
+            out.append(m.step_batch([(s, toks[at:at + c], _all(c))])[0])
+            at += c
+        assert m.seq_len(s) == n
+        assert _err(np.concatenate(out), want) < TOL_F32
+    finally:
+        m.close()
+
+
+def test_batches_of_unequal_requests_against_each_alone(tmp_path):
+    cfg = U.small_config()
+    P = U.random_weights(cfg, 4)
+    reqs = [U.tokens(n, cfg["vocab"], 10 + i) for i, n in enumerate((67, 5, 130, 31))]
+    want = [O.forward(cfg, P, t) for t in reqs]
+    # per step: (request, tokens taken) -- long portions beside single decode tokens, requests joining and pausing
+    plan = [[(0, 40), (1, 2)], [(0, 1), (1, 1), (2, 64)], [(2, 2), (0, 1), (3, 30)], [(1, 2), (2, 60), (3, 1), (0, 25)], [(2, 0)]]
+    m = _load(tmp_path, cfg, P)
+    try:
+        seqs = [m.seq_alloc() for _ in reqs]
+        at = [0] * len(reqs)
+        got = [[] for _ in reqs]
+        for step in plan:
+            step = [(r, c if c else len(reqs[r]) - at[r]) for r, c in step]
+            out, _ = m.step_batch([(seqs[r], reqs[r][at[r]:at[r] + c], _all(c)) for r, c in step])
+            row = 0
+            for r, c in step:
+                got[r].append(out[row:row + c])
+                row += c
+                at[r] += c
+        for r in range(len(reqs)):
+            have = np.concatenate(got[r])
+            assert _err(have, want[r][:len(have)]) < TOL_F32, r
+        assert at[2] == 130 and at[0] == 67
+    finally:
+        m.close()
+
+
+def test_pages_and_slots_that_are_freed_and_used_again(tmp_path):
+    cfg = U.small_config()
+    P = U.random_weights(cfg, 5)
+    m = _load(tmp_path, cfg, P, max_seq_len=192, kv_pool_tokens=256, max_seqs=2)        # 4 pages of 64, 2 slots
+    try:
+        for rnd in range(3):
+            reqs = [U.tokens(n, cfg["vocab"], 20 + 2 * rnd + i) for i, n in enumerate((100 + 7 * rnd, 90 - 11 * rnd))]
+            seqs = [m.seq_alloc(), m.seq_alloc()]
+            with pytest.raises(Exception):
+                m.seq_alloc()                                     # both slots taken
+            out, _ = m.step_batch([(seqs[0], reqs[0][:50], []), (seqs[1], reqs[1], _all(len(reqs[1])))])
+            assert _err(out, O.forward(cfg, P, reqs[1])) < TOL_F32
+            out, _ = m.step_batch([(seqs[0], reqs[0][50:], _all(len(reqs[0]) - 50))])
+            assert _err(out, O.forward(cfg, P, reqs[0])[50:]) < TOL_F32
+            assert m.active_kv_cache_bytes() > 0
+            for s in seqs:
+                m.seq_free(s)
+            assert m.active_kv_cache_bytes() == 0
+        # a step that does not fit in the pool fails and leaves the sequence as it was
+        a, b = m.seq_alloc(), m.seq_alloc()
+        m.step_batch([(a, U.tokens(150, cfg["vocab"], 1), None)])
+        with pytest.raises(Exception):
+            m.step_batch([(b, U.tokens(120, cfg["vocab"], 2), None)])
+        assert m.seq_len(b) == 0 and m.seq_len(a) == 150
+    finally:
+        m.close()
+
+
+@pytest.mark.parametrize("decoded", [False, True])
+@pytest.mark.parametrize("size", [20, 64, 5])
+def test_planted_keys_at_the_edges_of_the_window_and_at_page_borders(tmp_path, decoded, size):
+    cfg, P, QT, KT = U.planted_window(size)
+    m = _load(tmp_path, cfg, P)
+    try:
+        # (key position, query position): the window's last and first-outside position, keys on both sides of a page border (pages
+        # of 64 tokens), the same far into the sequence
+        cases = [(0, size - 1), (0, size), (1, size), (63, 64), (64, 65), (63, 63 + size - 1), (63, 63 + size), (64, 64 + size - 1), (64, 64 + size),
+                 (3, 199), (199 - size + 1, 199), (199 - size, 199), (127, 128), (128, 128 + size - 1), (128, 128 + size)]
+        for kp, qp in cases:
+            if not 0 <= kp < qp < 200:
+                continue
+            toks = U.tokens(200, 65, kp * 1000 + qp)
+            toks[kp], toks[qp] = KT, QT
+            want = O.forward(cfg, P, toks[:qp + 1])
+            plain = list(toks)
+            plain[kp] = (toks[kp - 1] + 1) % 65 if kp else 1
+            moved = float(np.abs(O.forward(cfg, P, plain[:qp + 1])[qp] - want[qp]).max() / np.abs(want[qp]).max())
+            seen = qp - kp < size
+            assert (moved > 0.1) == seen and (seen or moved < 0.01), (kp, qp, moved)       # the planted key matters exactly where the mask shows it
+            s = m.seq_alloc()
+            if decoded:
+                lo = max(1, qp - 2)
+                m.step_batch([(s, toks[:lo], [])])
+                got = np.concatenate([m.step_batch([(s, [toks[p]], [0])])[0] for p in range(lo, qp + 1)])
+                assert _err(got, want[lo:qp + 1]) < TOL_F32, (kp, qp)
+            else:
+                got, _ = m.step_batch([(s, toks[:qp + 1], [qp - 1, qp])])
+                assert _err(got, want[qp - 1:qp + 1]) < TOL_F32, (kp, qp)
+            m.seq_free(s)
+    finally:
+        m.close()
+
+
+@pytest.mark.parametrize("decoded", [False, True])
+def test_a_planted_key_far_back_among_hundreds_in_differential_attention(tmp_path, decoded):
+    cfg, P, QT, KT = U.planted_causal()
+    m = _load(tmp_path, cfg, P)
+    try:
+        for kp, qp in [(3, 290), (63, 300), (64, 257), (0, 449), (200, 449)]:
+            toks = U.tokens(450, 65, kp + qp)
+            toks[kp], toks[qp] = KT, QT
+            want = O.forward(cfg, P, toks[:qp + 1])
+            plain = list(toks); plain[kp] = 1
+            assert _err(O.forward(cfg, P, plain[:qp + 1])[qp], want[qp]) > 0.1
+            s = m.seq_alloc()
+            if decoded:
+                m.step_batch([(s, toks[:qp - 2], [])])
+                got = np.concatenate([m.step_batch([(s, [toks[p]], [0])])[0] for p in range(qp - 2, qp + 1)])
+                assert _err(got, want[qp - 2:qp + 1]) < TOL_F32, (kp, qp)
+            else:
+                got, _ = m.step_batch([(s, toks[:qp + 1], [qp - 1, qp])])
+                assert _err(got, want[qp - 1:qp + 1]) < TOL_F32, (kp, qp)
+            m.seq_free(s)
+    finally:
+        m.close()
+
+
+@pytest.mark.parametrize("kind", ["hgrn2", "parallel"])
+def test_a_token_long_ago_still_shows_through_the_recurrent_state(tmp_path, kind):
+    """Gates close to one: swapping token 2 moves the logits 250 tokens later, in the oracle and -- through a portion, a long run of
+    single tokens and another portion -- in the library."""
+    if kind == "hgrn2":
+        cfg = U.config([U.layer("hgrn2", U.hgrn(heads=2, dim=8, vdim=8), None)], vocab=37, width=24)
+        P = U.random_weights(cfg, 9)
+        P["l0.mix.lower"][:] = U.bf16_round(np.full(16, 0.99))
+        P["l0.mix.f.b"][:] = 3.0
+    else:
+        cfg = U.config([_par(U.left(size=8), U.right(heads=2, vdim=8, state=8, groups=1, conv=2, norm_groups=1), None, 0.2, 1.0)], vocab=37, width=24)
+        P = U.random_weights(cfg, 9)
+        P["l0.mix.right.A_log"][:] = -6.0
+        P["l0.mix.right.dt_bias"][:] = -1.0
+    toks = U.tokens(256, 37, 9)
+    other = list(toks); other[2] = (toks[2] + 5) % 37
+    want, want2 = O.forward(cfg, P, toks), O.forward(cfg, P, other)
+    assert _err(want2[255], want[255]) > 1.5e-3                   # several times what the comparison below allows
+    m = _load(tmp_path, cfg, P)
+    try:
+        for t, w in ((toks, want), (other, want2)):
+            s = m.seq_alloc()
+            m.step_batch([(s, t[:40], [])])
+            for p in range(40, 200):
+                m.step_batch([(s, [t[p]], [])], want_logits=False)
+            got, _ = m.step_batch([(s, t[200:], [54, 55])])
+            assert _err(got, w[254:256]) < TOL_F32
+            m.seq_free(s)
+    finally:
+        m.close()
+
+
+def test_first_tokens_of_a_sequence(tmp_path):
+    cfg = U.small_config()
+    P = U.random_weights(cfg, 8)
+    m = _load(tmp_path, cfg, P)
+    try:
+        for n in (1, 2, 3, 5):
+            toks = U.tokens(n, cfg["vocab"], 40 + n)
+            s = m.seq_alloc()
+            got, _ = m.step_batch([(s, toks, _all(n))])
+            assert _err(got, O.forward(cfg, P, toks)) < TOL_F32
+            m.seq_free(s)
+        # a fresh slot starts from zero states and an empty convolution tail although the one before it left its own behind
+        toks = U.tokens(4, cfg["vocab"], 50)
+        s = m.seq_alloc()
+        got = np.concatenate([m.step_batch([(s, [t], [0])])[0] for t in toks])
+        assert _err(got, O.forward(cfg, P, toks)) < TOL_F32
+    finally:
+        m.close()
+
+
+def test_long_decoding_past_many_windows(tmp_path):
+    cfg = U.small_config()                                        # windows of 20 / 33, query growth every 7 positions
+    P = U.random_weights(cfg, 9)
+    toks = U.tokens(230, cfg["vocab"], 9)
+    want = O.forward(cfg, P, toks)
+    m = _load(tmp_path, cfg, P)
+    try:
+        s = m.seq_alloc()
+        m.step_batch([(s, toks[:10], [])])
+        got = np.concatenate([m.step_batch([(s, [toks[p]], [0])])[0] for p in range(10, 230)])
+        assert _err(got, want[10:]) < TOL_F32
+    finally:
+        m.close()
+
+
+OTHER = {
+    "odd width, value size above key size, window of one page": U.config(
+        [_par(U.left(heads=2, kv_heads=1, dim=12, vdim=40, size=64, dims=6), U.right(heads=2, vdim=34, state=6, groups=1, conv=5, norm_groups=4), U.moe(), 1.0, 1.0)],
+        vocab=53, width=30, groups=5),
+    "window of one, scales of one, one head": U.config([_par(U.left(heads=1, kv_heads=1, dim=8, vdim=8, size=1), U.right(heads=1, vdim=8, state=8, groups=1), None, 1.0, 1.0)],
+                                                        groups=1),
+    "many heads mixed": U.config([_par(U.left(heads=20, kv_heads=4, dim=8, vdim=8, size=40, scale=0.3), U.right(heads=8, vdim=4, state=4, groups=4, conv=3, norm_groups=8),
+                                       U.moe(experts=7, top=3, ff=36, shared=24))], width=64, groups=4),
+    "forty heads mixed": U.config([_par(U.left(heads=40, kv_heads=8, dim=8, vdim=4, size=12, scale=0.3), U.right(), None)], width=64, groups=2),
+    "wide heads": U.config([_par(U.left(heads=2, kv_heads=1, dim=160, vdim=96, size=30, scale=0.05, dims=64), U.right(heads=1, vdim=48, state=144, groups=1), None),
+                            U.layer("attention", U.attn(heads=2, kv_heads=1, dim=96, vdim=144, scale=0.05), None), U.layer("hgrn2", U.hgrn(heads=1, dim=144, vdim=48), None)],
+                           width=72),
+    "no window reached": U.config([_par(U.left(size=500), U.right(), U.moe())]),
+    "a layer on a tensor-less layer's source, the first layer reused twice": U.config(
+        [U.layer("hgrn2", U.hgrn(), U.moe(shared=0)), U.layer("attention", U.attn(), None), U.layer("hgrn2", U.hgrn(), U.moe(shared=0), weights_of=0),
+         U.layer("hgrn2", U.hgrn(), U.moe(shared=0), weights_of=0), U.layer("attention", U.attn(), None, weights_of=1)]),
+    "seventy experts": U.config([U.layer("hgrn2", U.hgrn(), U.moe(experts=70, top=6, ff=8, shared=16))], width=32, groups=1),
+}
+
+
+@pytest.mark.parametrize("name", list(OTHER))
+def test_other_sizes_whole_portioned_and_decoded(tmp_path, name):
+    cfg = OTHER[name]
+    P = U.random_weights(cfg, 11)
+    toks = U.tokens(150, cfg["vocab"], 11)
+    want = O.forward(cfg, P, toks)
+    m = _load(tmp_path, cfg, P)
+    try:
+        a, b = m.seq_alloc(), m.seq_alloc()
+        whole, _ = m.step_batch([(a, toks, _all(150))])
+        assert _err(whole, want) < TOL_F32
+        out, at = [], 0
+        for c in [70, 2, 33, 1, 1, 17, 1, 25]:
+            out.append(m.step_batch([(b, toks[at:at + c], _all(c))])[0])
+            at += c
+        assert _err(np.concatenate(out), want) < TOL_F32
+    finally:
+        m.close()
+
+
+def test_greedy_generation_through_generate_and_through_the_engine(tmp_path):
+    from crane_amd.backend import GenerationConfig
+    from crane_amd.engine import GenerationParams, InferenceEngine
+    cfg = U.small_config()
+    P = U.random_weights(cfg, 12)
+    prompts = [U.tokens(n, cfg["vocab"], 60 + i) for i, n in enumerate((9, 70, 3, 25, 40))]
+    lens = [12, 6, 20, 9, 15]
+    want = [O.greedy(cfg, P, p, n) for p, n in zip(prompts, lens)]
+    m = _load(tmp_path, cfg, P, max_seq_len=128, kv_pool_tokens=384, max_seqs=4, prefill_chunk=48)
+    try:
+        assert m.generate(prompts[0], GenerationConfig.greedy(lens[0]))[len(prompts[0]):] == want[0]
+        m.clear_kv_cache()
+        eng = InferenceEngine(m, max_running=3)                   # 5 requests, 3 slots, 48-row steps: prompts are fed in portions
+        ids = [eng.submit(p, GenerationParams.greedy(n)) for p, n in zip(prompts, lens)]
+        toks, done = eng.run_until_idle()
+        for rid, w in zip(ids, want):
+            assert toks[rid] == w
+            assert done[rid].kind == "finished" and done[rid].finish_reason == "length"
+        st = eng.stats()
+        assert st["completed"] == 5 and st["failed"] == 0 and st["free_pages"] == st["total_pages"]
+        # sampled requests run through the same steps and the device sampler
+        rid = eng.submit(prompts[3], GenerationParams(max_tokens=8, temperature=0.8, top_p=0.9, top_k=20, seed=5))
+        toks, done = eng.run_until_idle()
+        assert len(toks[rid]) == 8 and all(0 <= t < cfg["vocab"] for t in toks[rid])
+        eng.close()
+    finally:
+        m.close()
+
+
+def test_bfloat16_format_against_the_oracle_and_across_schedules(tmp_path):
+    cfg = U.small_config()
+    P = U.random_weights(cfg, 13)
+    toks = U.tokens(100, cfg["vocab"], 13)
+    want = O.forward(cfg, P, toks)
+    m = _load(tmp_path, cfg, P, dtype="bfloat16")
+    try:
+        a, b = m.seq_alloc(), m.seq_alloc()
+        whole, _ = m.step_batch([(a, toks, _all(100))])
+        assert _err_most(whole, want) < TOL_BF16
+        out, at = [], 0
+        for c in [50, 2, 13, 1, 1, 33]:
+            out.append(m.step_batch([(b, toks[at:at + c], _all(c))])[0])
+            at += c
+        assert _err_most(np.concatenate(out), want) < TOL_BF16
+        assert _err_most(np.concatenate(out), whole) < TOL_BF16
+    finally:
+        m.close()
+
+
+def test_fork_carries_pages_states_and_convolution_tails(tmp_path):
+    cfg = U.small_config()
+    P = U.random_weights(cfg, 14)
+    toks = U.tokens(80, cfg["vocab"], 14)
+    want = O.forward(cfg, P, toks)
+    m = _load(tmp_path, cfg, P)
+    try:
+        a = m.seq_alloc()
+        m.step_batch([(a, toks[:37], [])])
+        b = m.seq_fork(a)
+        ga, _ = m.step_batch([(a, toks[37:], _all(43)), ])
+        gb, _ = m.step_batch([(b, toks[37:], _all(43))])
+        assert _err(ga, want[37:]) < TOL_F32 and _err(gb, want[37:]) < TOL_F32
+        with pytest.raises(Exception):
+            m.seq_truncate(a, 10)                                 # a recurrent state cannot be rewound
+    finally:
+        m.close()
+
+
+def test_synthetic_registry_model_generates(tmp_path):
+    from crane_amd import configs
+    from crane_amd.backend import GenerationConfig, Model
+    m = Model.synthetic(configs.get_config("tiny-nevotar"), seed=3, max_seq_len=128, max_seqs=2)
+    try:
+        assert m.num_layers() == 5 and m.vocab_size == 320
+        out = m.generate([1, 2, 3, 4, 5], GenerationConfig.greedy(6))
+        assert len(out) == 11
+        logits = m.forward_step([7, 8, 9], 0)[0, 0]
+        assert np.isfinite(logits).all() and int(np.argmax(logits)) == m.forward_step_greedy([7, 8, 9], 0)
+        assert m.decode_bytes_per_token(64) > m.weight_bytes() // 8
+    finally:
+        m.close()
+
+
+def _wide_config(window=96):
+    """Sizes the matrix-core kernels take (head sizes multiples of 16, wide products)."""
+    return U.config([U.layer("attention", U.attn(heads=4, kv_heads=2, dim=32, vdim=48, every=64, scale=0.2), U.moe(experts=6, top=2, ff=128, shared=128)),
+                     _par(U.left(heads=4, kv_heads=2, dim=32, vdim=48, size=window, scale=0.2), U.right(heads=4, vdim=32, state=32, groups=2, conv=4, norm_groups=2),
+                          U.moe(experts=4, top=1, ff=128, shared=0)),
+                     U.layer("hgrn2", U.hgrn(heads=2, dim=32, vdim=64), None),
+                     U.layer("attention", U.attn(heads=4, kv_heads=2, dim=32, vdim=48, every=64, scale=0.2), U.moe(experts=6, top=2, ff=128, shared=128), weights_of=0)],
+                    vocab=256, width=128, groups=2)
+
+
+@pytest.mark.parametrize("dtype,tol,err", [("float32", TOL_F32, _err), ("bfloat16", TOL_BF16, _err_long)])
+def test_decode_steps_over_hundreds_of_keys_and_a_long_portion_in_chunks(tmp_path, dtype, tol, err):
+    cfg = _wide_config(window=300)
+    P = U.random_weights(cfg, 15)
+    toks = U.tokens(460, cfg["vocab"], 15)
+    want = O.forward(cfg, P, toks)
+    m = _load(tmp_path, cfg, P, dtype=dtype)
+    try:
+        a, b = m.seq_alloc(), m.seq_alloc()
+        whole, _ = m.step_batch([(a, toks, _all(460))])               # chunk-parallel recurrences, matrix-core differential attention (bfloat16)
+        assert err(whole, want) < tol
+        m.step_batch([(b, toks[:430], [])])
+        tail = np.concatenate([m.step_batch([(b, [t], [0])])[0] for t in toks[430:]])     # split keys: a window of 300, 430 causal keys
+        assert err(tail, want[430:]) < tol
+    finally:
+        m.close()
+
+
+def test_a_step_larger_than_one_pass_is_cut_into_passes(tmp_path):
+    cfg = U.small_config()
+    P = U.random_weights(cfg, 16)
+    reqs = [U.tokens(n, cfg["vocab"], 70 + i) for i, n in enumerate((75, 3, 41))]
+    want = [O.forward(cfg, P, t) for t in reqs]
+    m = _load(tmp_path, cfg, P, prefill_chunk=32)
+    try:
+        seqs = [m.seq_alloc() for _ in reqs]
+        out, _ = m.step_batch([(s, t, _all(len(t))) for s, t in zip(seqs, reqs)])
+        assert _err(out, np.concatenate(want)) < TOL_F32
+    finally:
+        m.close()
+
+
+def test_matrix_core_attention_of_prompt_passes_against_the_plain_kernel(tmp_path):
+    cfg = _wide_config()
+    P = U.random_weights(cfg, 17)
+    toks = U.tokens(300, cfg["vocab"], 17)
+    want = O.forward(cfg, P, toks)
+    m = _load(tmp_path, cfg, P, dtype="bfloat16")
+    try:
+        a, b = m.seq_alloc(), m.seq_alloc()
+        fast, _ = m.step_batch([(a, toks[:130], _all(130))])
+        fast2, _ = m.step_batch([(a, toks[130:], _all(170))])        # a portion whose keys lie in earlier pages
+        fast = np.concatenate([fast, fast2])
+        m.debug_set("lay_attn_mfma", 0)
+        plain, _ = m.step_batch([(b, toks, _all(300))])
+        assert _err_most(fast, want) < TOL_BF16 and _err_most(plain, want) < TOL_BF16
+        assert _err_most(fast, plain) < 2e-2
+    finally:
+        m.close()
+
+
+def _drawn_config(seed):
+    """A model of this design with layer order, sizes, windows and constants drawn from the seed."""
+    rs = np.random.RandomState(200 + seed)
+    pick = lambda *xs: xs[rs.randint(len(xs))]
+    width, layers = pick(96, 120, 192, 240), []
+
+    def mlp():
+        if rs.rand() < 0.25:
+            return None
+        ex = pick(2, 3, 5, 8)
+        return U.moe(experts=ex, top=rs.randint(1, min(ex, 3) + 1), ff=pick(32, 96, 136), limit=pick(0.5, 1.0, 7.0), shared=pick(0, 64, 128), shared_limit=pick(1.0, 2.5))
+
+    for _ in range(rs.randint(2, 5)):
+        kind = pick("attention", "hgrn2", "parallel")
+        kvh = pick(1, 2, 4)
+        if kind == "attention":
+            mx = U.attn(heads=kvh * pick(1, 2, 3), kv_heads=kvh, dim=pick(16, 24, 32, 64), vdim=pick(16, 32, 48, 80), diff=pick(0.1, 0.5, 0.8), coef=pick(0.0, 0.1, 0.4),
+                        every=pick(1, 16, 50, 64), scale=pick(0.1, 0.2))
+        elif kind == "hgrn2":
+            mx = U.hgrn(heads=pick(1, 2, 4), dim=pick(8, 16, 32, 64), vdim=pick(16, 32, 72))
+        else:
+            dim = pick(16, 24, 32, 64)
+            gr = pick(1, 2)
+            heads = gr * pick(1, 2, 3)
+            vd = pick(8, 16, 24)
+            mx = U.side(U.left(heads=kvh * pick(1, 2, 3), kv_heads=kvh, dim=dim, vdim=pick(16, 32, 48, 72), size=pick(17, 40, 64, 80, 128), dims=pick(dim, dim // 2, dim // 4 * 2),
+                               base=pick(100.0, 10000.0, 1000000.0), scale=pick(0.1, 0.2)),
+                        U.right(heads=heads, vdim=vd, state=pick(8, 16, 32), groups=gr, conv=pick(2, 3, 4), norm_groups=pick(1, heads)), pick(0.5, 0.8, 1.0), pick(0.7, 1.1, 1.0))
+        layers.append(U.layer(kind, mx, mlp()))
+    n = len(layers)
+    for k in range(rs.randint(0, 3)):                             # some layers run once more, on the same tensors
+        j = rs.randint(n)
+        layers.append(dict(layers[j], weights_of=j))
+    return U.config(layers, vocab=pick(97, 256, 601), width=width, eps=pick(1e-6, 1e-5, 1e-4), groups=pick(1, 2, 3, 4))
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_drawn_models_whole_in_portions_and_decoded_in_both_formats(tmp_path, seed):
+    cfg = _drawn_config(seed)
+    P = U.random_weights(cfg, 30 + seed)
+    toks = U.tokens(170, cfg["vocab"], 30 + seed)
+    want = O.forward(cfg, P, toks)
+    for dtype, tol, err in (("float32", TOL_F32, _err), ("bfloat16", TOL_BF16, _err_most)):
+        m = _load(tmp_path, cfg, P, dtype=dtype)
+        try:
+            a, b = m.seq_alloc(), m.seq_alloc()
+            whole, _ = m.step_batch([(a, toks, _all(170))])
+            assert err(whole, want) < tol, (dtype, "whole")
+            out, at = [], 0
+            for c in [70, 2, 33, 1, 1, 17, 1, 25, 1, 1, 18]:
+                out.append(m.step_batch([(b, toks[at:at + c], _all(c))])[0])
+                at += c
+            assert at == 170 and err(np.concatenate(out), want) < tol, (dtype, "portions")
+        finally:
+            m.close()
