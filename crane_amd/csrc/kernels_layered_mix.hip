@@ -344,26 +344,217 @@ __global__ __launch_bounds__(256) void lay_attn_talk_kernel(LAttnArgs a, const f
         }
     }
 }
-// merge of the splits (single-token portions: the tile's rows are the H heads); one block per sequence
-__global__ __launch_bounds__(256) void lay_attn_talk_merge_kernel(LAttnArgs a, int nsplit) {
+// merge of the splits (single-token portions: the tile's rows are the H heads); one block of 64 threads per (sequence, head): the
+// splits' factors e^(m_z - M) are formed once (one lane each, up to 64 splits), then a thread per output element sums
+constexpr int LT_MAX_SPLIT = 64;
+__global__ __launch_bounds__(64) void lay_attn_talk_merge_kernel(LAttnArgs a, int nsplit) {
+    __shared__ float wz[LT_MAX_SPLIT];
     const LaySegDev sg = a.segs[blockIdx.x];
-    const int H = a.H, e = a.e;
-    const size_t t0 = (size_t)blockIdx.x * nsplit * H;
-    for (int idx = threadIdx.x; idx < H * e; idx += 256) {
-        const int h = idx / e, i = idx - h * e;
-        float M = -INFINITY;
-        for (int z = 0; z < nsplit; ++z) M = fmaxf(M, a.part_ml[(t0 + (size_t)z * H + h) * 2]);
-        float L = 0.f, acc = 0.f;
-        for (int z = 0; z < nsplit; ++z) {
-            const size_t pr = t0 + (size_t)z * H + h;
-            const float mz = a.part_ml[pr * 2];
-            const float wgt = mz == -INFINITY ? 0.f : expf(mz - M);
-            L = fmaf(a.part_ml[pr * 2 + 1], wgt, L);
-            acc = fmaf(a.part_o[pr * e + i], wgt, acc);
-        }
-        a.out[(size_t)sg.row0 * a.ldo + h * e + i] = acc / L * a.out_scale;
+    const int H = a.H, e = a.e, h = blockIdx.y, lane = threadIdx.x;
+    const size_t t0 = (size_t)blockIdx.x * nsplit * H + h;
+    const float mz = lane < nsplit ? a.part_ml[(t0 + (size_t)lane * H) * 2] : -INFINITY;
+    const float M = wave_max(mz);
+    const float wgt = mz == -INFINITY ? 0.f : expf(mz - M);
+    const float L = wave_sum(lane < nsplit ? a.part_ml[(t0 + (size_t)lane * H) * 2 + 1] * wgt : 0.f);
+    wz[lane] = wgt;
+    __syncthreads();
+    const float inv = a.out_scale / L;
+    for (int i = lane; i < e; i += 64) {
+        float acc = 0.f;
+        for (int z = 0; z < nsplit; ++z) acc = fmaf(a.part_o[(t0 + (size_t)z * H) * e + i], wz[z], acc);
+        a.out[(size_t)sg.row0 * a.ldo + h * e + i] = acc * inv;
     }
 }
+// Matrix-core form for prompt passes in the bfloat16 format (key and value sizes multiples of 16 up to 128, up to 16 heads): a
+// block owns 16 positions of one sequence, one wave per head.  Per tile of 64 keys every wave forms S_h = Q_h K^T on
+// v_mfma_f32_16x16x16_bf16 from the bf16-rounded q and the cached keys of its key head and leaves it, scaled, in LDS; after a
+// barrier it mixes the H raw scores of each of its (position, key) places with its line of the matrix in the accumulator's own
+// layout (A[i = lane % 16][k = 4 (lane / 16) ..], B[k][j = lane % 16], D[i = 4 (lane / 16) + r][j = lane % 16]); mask, running
+// max / sum and the weights are f32, the weights enter P V as a bf16 hi + lo pair (two products per tile).
+constexpr int LTM_KT = 64, LTM_LDS = 68;          // keys per tile; f32 stride of a raw-score row (68: the two half-waves of a read hit disjoint banks)
+static size_t lay_talk_mfma_lds(int H, int G, int d, int e) {
+    return (size_t)(G * LTM_KT * (d + 8) + G * e * (LTM_KT + 8) + 2 * H * 16 * (LTM_KT + 8)) * sizeof(uint16_t) +
+           (size_t)(H * 16 * LTM_LDS + H * H) * sizeof(float);
+}
+template <int NDMAX, int NEMAX, int NT>
+__global__ __launch_bounds__(NT) void lay_attn_talk_mfma_kernel(LAttnArgs a, const float* __restrict__ talk) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
+    const int d = a.d, e = a.e, H = a.H, G = a.G, nrep = H / G;
+    const int ldq = d + 8, ldp = LTM_KT + 8;
+    uint16_t* Ks = smem;                               // [G][64][d + 8]
+    uint16_t* Vt = Ks + G * LTM_KT * ldq;              // [G][e][72] the value tiles transposed (the B operand of P V: 4 keys of one element)
+    uint16_t* Ph = Vt + G * e * ldp;                   // [H][16][72] hi
+    uint16_t* Pl = Ph + H * 16 * ldp;                  // ... lo
+    float* Sr = (float*)(Pl + H * 16 * ldp);           // [H][16][68] raw scores of every head
+    float* tk = Sr + H * 16 * LTM_LDS;                 // [H][H]
+    const LaySegDev sg = a.segs[blockIdx.x];
+    const int p0 = (int)blockIdx.y * 16;
+    if (p0 >= sg.n) return;
+    const int np = min(16, sg.n - p0);
+    const int tid = threadIdx.x, nt = 64 * H, lane = tid & 63, h = tid >> 6, lr = lane & 15, lg = lane >> 4;
+    const int g = h / nrep;
+    const int win = (int)min(a.win, 1ll << 30);
+    for (int idx = tid; idx < H * H; idx += nt) tk[idx] = talk[idx];
+    // this lane's part of the q fragments: position p0 + lr, elements kk 16 + 4 lg .. + 3 of head h
+    const int nd = d / 16, ne = e / 16;
+    bf16x4 qf[NDMAX];
+#pragma unroll
+    for (int kk = 0; kk < NDMAX; ++kk) {
+        qf[kk] = (bf16x4){0, 0, 0, 0};
+        if (kk < nd && lr < np) {
+            const float4 x = *(const float4*)(a.proj + (size_t)(sg.row0 + p0 + lr) * a.ldp + a.q_off + h * d + kk * 16 + 4 * lg);
+            const uint32_t lo = pack_bf16x2(x.x, x.y), hi = pack_bf16x2(x.z, x.w);
+            qf[kk] = (bf16x4){(short)(lo & 0xFFFFu), (short)(lo >> 16), (short)(hi & 0xFFFFu), (short)(hi >> 16)};
+        }
+    }
+    int qpos[4]; bool qok[4];
+    float m[4] = {-INFINITY, -INFINITY, -INFINITY, -INFINITY}, l[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int r = 0; r < 4; ++r) { qok[r] = 4 * lg + r < np; qpos[r] = sg.start_pos + p0 + 4 * lg + r; }
+    const int pmin = sg.start_pos + p0, pmax = pmin + np - 1;
+    const int main_lo = max(0, pmin - win + 1);
+    const int total = pmax - main_lo + 1;
+    f32x4 O[NEMAX];
+#pragma unroll
+    for (int n = 0; n < NEMAX; ++n) O[n] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    uint16_t* ph = Ph + h * 16 * ldp;
+    uint16_t* pl = Pl + h * 16 * ldp;
+    const uint16_t* kg = Ks + g * LTM_KT * ldq;
+    const uint16_t* vg = Vt + g * e * ldp;
+    float* sr = Sr + h * 16 * LTM_LDS;
+    for (int v0 = 0; v0 < total; v0 += LTM_KT) {
+        __syncthreads();                   // the previous tile is consumed: keys, values and raw scores may be replaced
+        for (int idx = tid; idx < G * LTM_KT * (d / 8); idx += nt) {
+            const int rw = idx / (d / 8), i = (idx - rw * (d / 8)) * 8, kgi = rw / LTM_KT, sl = rw - kgi * LTM_KT, v = v0 + sl;
+            u32x4 pk = {0u, 0u, 0u, 0u};
+            if (v < total) {
+                const int j = main_lo + v;
+                const size_t row = ((size_t)a.bt[sg.bt_off + j / a.page] * G + kgi) * a.page + (size_t)(j % a.page);
+                pk = *(const u32x4*)((const uint16_t*)a.kpool + row * d + i);
+            }
+            *(u32x4*)&Ks[(size_t)rw * ldq + i] = pk;
+        }
+        for (int idx = tid; idx < G * LTM_KT * (e / 8); idx += nt) {
+            const int rw = idx / (e / 8), i = (idx - rw * (e / 8)) * 8, kgi = rw / LTM_KT, sl = rw - kgi * LTM_KT, v = v0 + sl;
+            u32x4 pk = {0u, 0u, 0u, 0u};
+            if (v < total) {
+                const int j = main_lo + v;
+                const size_t row = ((size_t)a.bt[sg.bt_off + j / a.page] * G + kgi) * a.page + (size_t)(j % a.page);
+                pk = *(const u32x4*)((const uint16_t*)a.vpool + row * e + i);
+            }
+            uint16_t* vt = Vt + ((size_t)kgi * e + i) * ldp + sl;
+            vt[0] = (uint16_t)(pk.x & 0xFFFFu); vt[ldp] = (uint16_t)(pk.x >> 16);
+            vt[2 * ldp] = (uint16_t)(pk.y & 0xFFFFu); vt[3 * ldp] = (uint16_t)(pk.y >> 16);
+            vt[4 * ldp] = (uint16_t)(pk.z & 0xFFFFu); vt[5 * ldp] = (uint16_t)(pk.z >> 16);
+            vt[6 * ldp] = (uint16_t)(pk.w & 0xFFFFu); vt[7 * ldp] = (uint16_t)(pk.w >> 16);
+        }
+        __syncthreads();
+        f32x4 S[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) S[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int kk = 0; kk < NDMAX; ++kk) {
+            if (kk < nd) {
+                const bf16x4 qa = qf[kk];
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    const bf16x4 kb = *(const bf16x4*)&kg[(t * 16 + lr) * ldq + kk * 16 + 4 * lg];
+                    S[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(qa, kb, S[t], 0, 0, 0);
+                }
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) sr[(4 * lg + r) * LTM_LDS + t * 16 + lr] = S[t][r] * a.scale;
+        __syncthreads();                   // every head's raw scores are in LDS
+#pragma unroll
+        for (int t = 0; t < 4; ++t) S[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        for (int g2 = 0; g2 < H; ++g2) {
+            const float w = tk[h * H + g2];
+            const float* so = Sr + (size_t)g2 * 16 * LTM_LDS;
+#pragma unroll
+            for (int t = 0; t < 4; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) S[t][r] = fmaf(w, so[(4 * lg + r) * LTM_LDS + t * 16 + lr], S[t][r]);
+        }
+        float corr[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            float sc[4], tmax = -INFINITY;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const int v = v0 + t * 16 + lr, j = main_lo + v;
+                const bool vis = qok[r] && v < total && j <= qpos[r] && qpos[r] - j < win;
+                sc[t] = vis ? S[t][r] : -INFINITY;
+                tmax = fmaxf(tmax, sc[t]);
+            }
+            tmax = row16_max(tmax);
+            const float mn = fmaxf(m[r], tmax);
+            corr[r] = mn == -INFINITY ? 1.f : __expf(m[r] - mn);
+            float psum = 0.f;
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                const float p = sc[t] == -INFINITY ? 0.f : __expf(sc[t] - mn);
+                psum += p;
+                const uint16_t hi = f32_to_bf16(p);
+                ph[(4 * lg + r) * ldp + t * 16 + lr] = hi;
+                pl[(4 * lg + r) * ldp + t * 16 + lr] = f32_to_bf16(p - bf16_to_f32(hi));
+            }
+            psum = row16_sum(psum);
+            l[r] = l[r] * corr[r] + psum;
+            m[r] = mn;
+        }
+#pragma unroll
+        for (int n = 0; n < NEMAX; ++n)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) O[n][r] *= corr[r];
+        __syncthreads();                   // the wave's weights are in LDS
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+            const bf16x4 ah = *(const bf16x4*)&ph[lr * ldp + ks * 16 + 4 * lg];
+            const bf16x4 al = *(const bf16x4*)&pl[lr * ldp + ks * 16 + 4 * lg];
+#pragma unroll
+            for (int n = 0; n < NEMAX; ++n) {
+                if (n < ne) {
+                    const bf16x4 vb = *(const bf16x4*)&vg[(n * 16 + lr) * ldp + ks * 16 + 4 * lg];
+                    O[n] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(ah, vb, O[n], 0, 0, 0);
+                    O[n] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(al, vb, O[n], 0, 0, 0);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        if (!qok[r]) continue;
+        const float inv = a.out_scale / l[r];
+#pragma unroll
+        for (int n = 0; n < NEMAX; ++n)
+            if (n < ne) a.out[(size_t)(sg.row0 + p0 + 4 * lg + r) * a.ldo + h * e + n * 16 + lr] = O[n][r] * inv;
+    }
+}
+bool lay_attn_talk_mfma_fits(int H, int G, int d, int e) {
+    return H > 0 && H <= 16 && G > 0 && H % G == 0 && d > 0 && e > 0 && d % 16 == 0 && e % 16 == 0 && d <= 128 && e <= 128 &&
+           lay_talk_mfma_lds(H, G, d, e) <= LT_LDS_MAX;
+}
+template <int NT>
+static void lay_attn_talk_mfma_go(const LAttnArgs& a, const float* talk, dim3 grid, size_t lds, hipStream_t s) {
+    static bool raised = false;            // per instantiation
+    if (!raised) {
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&lay_attn_talk_mfma_kernel<8, 8, NT>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  (int)LT_LDS_MAX);
+        raised = true;
+    }
+    hipLaunchKernelGGL((lay_attn_talk_mfma_kernel<8, 8, NT>), grid, dim3((unsigned)(64 * a.H)), lds, s, a, talk);
+}
+void launch_lay_attn_talk_mfma(const LAttnArgs& a, const float* talk, int nseg, int max_n, hipStream_t s) {
+    if (nseg <= 0 || max_n <= 0) return;
+    const dim3 grid((unsigned)nseg, (unsigned)((max_n + 15) / 16));
+    const size_t lds = lay_talk_mfma_lds(a.H, a.G, a.d, a.e);
+    if (a.H <= 8) lay_attn_talk_mfma_go<512>(a, talk, grid, lds, s);
+    else lay_attn_talk_mfma_go<1024>(a, talk, grid, lds, s);
+}
+
 template <int KVT, int RPG, int NACC>
 static void lay_attn_talk_go(const LAttnArgs& a, const float* talk, int BQ, dim3 grid, size_t lds, hipStream_t s) {
     if (lds > LT_LDS_PLAIN) {
@@ -403,12 +594,12 @@ void launch_lay_attn_talk(const LAttnArgs& a0, const float* talk, int nseg, int 
             if (lay_talk_lds(H, a.G, a.d, a.e, bq) <= LT_LDS_MAX) { rpg = tr; BQ = bq; break; }
         }
     }
-    const int nsplit = (max_n == 1 && a.part_o && a.part_ml && a.nsplit > 1) ? a.nsplit : 1;
+    const int nsplit = (max_n == 1 && a.part_o && a.part_ml && a.nsplit > 1) ? std::min(a.nsplit, LT_MAX_SPLIT) : 1;
     const dim3 grid((unsigned)nseg, (unsigned)((max_n + BQ - 1) / BQ), (unsigned)nsplit);
     const size_t lds = lay_talk_lds(H, a.G, a.d, a.e, BQ);
     if (kvt == KV_F32) lay_attn_talk_r<KV_F32>(a, talk, rpg, BQ, grid, lds, s);
     else lay_attn_talk_r<KV_BF16>(a, talk, rpg, BQ, grid, lds, s);
-    if (nsplit > 1) hipLaunchKernelGGL(lay_attn_talk_merge_kernel, dim3((unsigned)nseg), dim3(256), 0, s, a, nsplit);
+    if (nsplit > 1) hipLaunchKernelGGL(lay_attn_talk_merge_kernel, dim3((unsigned)nseg, (unsigned)H), dim3(64), 0, s, a, nsplit);
 }
 
 }  // namespace cm

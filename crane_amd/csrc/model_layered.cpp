@@ -1587,7 +1587,11 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                                 a.nsplit = std::max(1, std::min({32, key_tiles, 256 / std::max(1, nseg), Layered::ATT_PARTS * 16 / std::max(1, nseg * H)}));
                                 a.part_o = L.att_po; a.part_ml = L.att_pml;
                             }
-                            launch_lay_attn_talk(a, sw.talk, nseg, max_n, kv_mode, s);
+                            if (L.attn_mfma && kv_mode == KV_BF16 && !all_decode && max_n >= 16 && lay_attn_talk_mfma_fits(H, G, d, e) && w.in_rows % 4 == 0 &&
+                                sw.q_off % 4 == 0)      // (16-byte loads of the query rows)
+                                launch_lay_attn_talk_mfma(a, sw.talk, nseg, max_n, s);
+                            else
+                                launch_lay_attn_talk(a, sw.talk, nseg, max_n, kv_mode, s);
                         } else if (sd.mixer == LMIX_SSM) {
                             const int N = sd.state, C = H * e + 2 * sd.groups * N;
                             LConvArgs c;
