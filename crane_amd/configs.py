@@ -273,7 +273,7 @@ CONFIGS.update({
 # ---- layer-list decoders: Nevotar ------------------------------------------------------------------------------------------
 def nevotar_config(vocab: int, width: int, kinds: "list | tuple", heads: int, kv_heads: int, dim: int, vdim: int, window: int,
                    rec_heads: int, rec_dim: int, rec_vdim: int, ssm_heads: int, ssm_vdim: int, state: int, ssm_groups: int, experts: int,
-                   top: int, expert_ff: int, shared_ff: int = 0, limit: float = 7.0, diff: float = 0.6, q_coef: float = 0.1, q_every: int = 1024,
+                   top: int, expert_ff: int, shared_ff: int = 0, limit: float = 7.0, diff: float = 0.5, q_coef: float = 0.1, q_every: int = 1024,
                    rot_dims: "int | None" = None, rot_base: float = 1000000.0, conv: int = 4, ssm_norm_groups: int = 1, left_scale: float = 1.0,
                    right_scale: float = 1.0, norm_groups: int = 1, eps: float = 1e-6, no_ff: "tuple | list" = (), weights_of: "dict | None" = None) -> dict:
     """Pre-norm layers of the kinds named in `kinds`: "attention" (two softmax maps per head, `dim` per map), "hgrn2" (gated

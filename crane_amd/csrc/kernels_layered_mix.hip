@@ -422,31 +422,61 @@ __global__ __launch_bounds__(NT) void lay_attn_talk_mfma_kernel(LAttnArgs a, con
     const uint16_t* kg = Ks + g * LTM_KT * ldq;
     const uint16_t* vg = Vt + g * e * ldp;
     float* sr = Sr + h * 16 * LTM_LDS;
-    for (int v0 = 0; v0 < total; v0 += LTM_KT) {
-        __syncthreads();                   // the previous tile is consumed: keys, values and raw scores may be replaced
-        for (int idx = tid; idx < G * LTM_KT * (d / 8); idx += nt) {
-            const int rw = idx / (d / 8), i = (idx - rw * (d / 8)) * 8, kgi = rw / LTM_KT, sl = rw - kgi * LTM_KT, v = v0 + sl;
-            u32x4 pk = {0u, 0u, 0u, 0u};
-            if (v < total) {
-                const int j = main_lo + v;
-                const size_t row = ((size_t)a.bt[sg.bt_off + j / a.page] * G + kgi) * a.page + (size_t)(j % a.page);
-                pk = *(const u32x4*)((const uint16_t*)a.kpool + row * d + i);
-            }
-            *(u32x4*)&Ks[(size_t)rw * ldq + i] = pk;
+    // the cached row of every key of a tile (key head 0; -1 past the end), looked up one tile ahead so that the tile's loads do not
+    // wait for the page table
+    __shared__ int rowb[2][LTM_KT];
+    auto look_up = [&](int v0, int buf) {
+        if (tid < LTM_KT) {
+            const int v = v0 + tid, j = main_lo + v;
+            rowb[buf][tid] = v < total ? a.bt[sg.bt_off + j / a.page] * G * a.page + j % a.page : -1;
         }
-        for (int idx = tid; idx < G * LTM_KT * (e / 8); idx += nt) {
-            const int rw = idx / (e / 8), i = (idx - rw * (e / 8)) * 8, kgi = rw / LTM_KT, sl = rw - kgi * LTM_KT, v = v0 + sl;
-            u32x4 pk = {0u, 0u, 0u, 0u};
-            if (v < total) {
-                const int j = main_lo + v;
-                const size_t row = ((size_t)a.bt[sg.bt_off + j / a.page] * G + kgi) * a.page + (size_t)(j % a.page);
-                pk = *(const u32x4*)((const uint16_t*)a.vpool + row * e + i);
+    };
+    look_up(0, 0);
+    const int nk = G * LTM_KT * (d / 8), nv = G * LTM_KT * (e / 8);
+    for (int v0 = 0, buf = 0; v0 < total; v0 += LTM_KT, buf ^= 1) {
+        __syncthreads();                   // the previous tile is consumed: keys, values and raw scores may be replaced
+        look_up(v0 + LTM_KT, buf ^ 1);
+        // four independent 16-byte loads in flight per thread, then their stores
+        for (int base = 0; base < nk; base += 4 * nt) {
+            u32x4 pk[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int idx = base + c * nt + tid;
+                pk[c] = (u32x4){0u, 0u, 0u, 0u};
+                if (idx < nk) {
+                    const int rw = idx / (d / 8), i = (idx - rw * (d / 8)) * 8, kgi = rw / LTM_KT, rb = rowb[buf][rw - kgi * LTM_KT];
+                    if (rb >= 0) pk[c] = *(const u32x4*)((const uint16_t*)a.kpool + ((size_t)rb + (size_t)kgi * a.page) * d + i);
+                }
             }
-            uint16_t* vt = Vt + ((size_t)kgi * e + i) * ldp + sl;
-            vt[0] = (uint16_t)(pk.x & 0xFFFFu); vt[ldp] = (uint16_t)(pk.x >> 16);
-            vt[2 * ldp] = (uint16_t)(pk.y & 0xFFFFu); vt[3 * ldp] = (uint16_t)(pk.y >> 16);
-            vt[4 * ldp] = (uint16_t)(pk.z & 0xFFFFu); vt[5 * ldp] = (uint16_t)(pk.z >> 16);
-            vt[6 * ldp] = (uint16_t)(pk.w & 0xFFFFu); vt[7 * ldp] = (uint16_t)(pk.w >> 16);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int idx = base + c * nt + tid;
+                if (idx < nk) { const int rw = idx / (d / 8), i = (idx - rw * (d / 8)) * 8; *(u32x4*)&Ks[(size_t)rw * ldq + i] = pk[c]; }
+            }
+        }
+        for (int base = 0; base < nv; base += 4 * nt) {
+            u32x4 pk[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int idx = base + c * nt + tid;
+                pk[c] = (u32x4){0u, 0u, 0u, 0u};
+                if (idx < nv) {
+                    const int rw = idx / (e / 8), i = (idx - rw * (e / 8)) * 8, kgi = rw / LTM_KT, rb = rowb[buf][rw - kgi * LTM_KT];
+                    if (rb >= 0) pk[c] = *(const u32x4*)((const uint16_t*)a.vpool + ((size_t)rb + (size_t)kgi * a.page) * e + i);
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int idx = base + c * nt + tid;
+                if (idx < nv) {
+                    const int rw = idx / (e / 8), i = (idx - rw * (e / 8)) * 8, kgi = rw / LTM_KT, sl = rw - kgi * LTM_KT;
+                    uint16_t* vt = Vt + ((size_t)kgi * e + i) * ldp + sl;
+                    vt[0] = (uint16_t)(pk[c].x & 0xFFFFu); vt[ldp] = (uint16_t)(pk[c].x >> 16);
+                    vt[2 * ldp] = (uint16_t)(pk[c].y & 0xFFFFu); vt[3 * ldp] = (uint16_t)(pk[c].y >> 16);
+                    vt[4 * ldp] = (uint16_t)(pk[c].z & 0xFFFFu); vt[5 * ldp] = (uint16_t)(pk[c].z >> 16);
+                    vt[6 * ldp] = (uint16_t)(pk[c].w & 0xFFFFu); vt[7 * ldp] = (uint16_t)(pk[c].w >> 16);
+                }
+            }
         }
         __syncthreads();
         f32x4 S[4];
