@@ -1262,31 +1262,68 @@ __global__ __launch_bounds__(LM_NT) void lay_attn_mfma_kernel(LAttnArgs a) {
 #pragma unroll
     for (int kk = 0; kk < NDMAX; ++kk)
         qf[kk] = kk < nd ? *(const bf16x4*)&Qs[(wave * 16 + lr) * ldq + kk * 16 + 4 * lg] : (bf16x4){0, 0, 0, 0};
-    for (int v0 = 0; v0 < total; v0 += LM_KT) {
+    // the cached rows behind the entries of a tile's key walk (null past the end), looked up one tile ahead so that the tile's loads
+    // do not wait for the page table
+    __shared__ LaRow rowp[2][LM_KT];
+    auto look_up = [&](int v0, int buf) {
+        if (tid < LM_KT) {
+            const int v = v0 + tid;
+            rowp[buf][tid] = v < total ? la_row<2>(a, sg, g, v, sink_hi, main_lo, pool) : LaRow{nullptr, nullptr};
+        }
+    };
+    auto transposed = [&](const u32x4& pk, int i, int sl) {
+        uint16_t* kt = Kt + i * ldp + sl;
+        kt[0] = (uint16_t)(pk.x & 0xFFFFu); kt[ldp] = (uint16_t)(pk.x >> 16);
+        kt[2 * ldp] = (uint16_t)(pk.y & 0xFFFFu); kt[3 * ldp] = (uint16_t)(pk.y >> 16);
+        kt[4 * ldp] = (uint16_t)(pk.z & 0xFFFFu); kt[5 * ldp] = (uint16_t)(pk.z >> 16);
+        kt[6 * ldp] = (uint16_t)(pk.w & 0xFFFFu); kt[7 * ldp] = (uint16_t)(pk.w >> 16);
+    };
+    look_up(0, 0);
+    const int nkl = LM_KT * (d / 8), nvl = LM_KT * (e / 8);
+    for (int v0 = 0, buf = 0; v0 < total; v0 += LM_KT, buf ^= 1) {
         __syncthreads();                   // previous tile consumed (first round: q fragments read, Qs free for Kt)
-        for (int idx = tid; idx < LM_KT * (d / 8); idx += LM_NT) {
-            const int sl = idx / (d / 8), i = (idx - sl * (d / 8)) * 8;
-            const int v = v0 + sl;
-            u32x4 pk = {0u, 0u, 0u, 0u};
-            if (v < total) pk = *(const u32x4*)((const uint16_t*)la_row<2>(a, sg, g, v, sink_hi, main_lo, pool).k + i);
-            *(u32x4*)&Ks[sl * ldq + i] = pk;
-            if (!WIDE && !ownv && i < e) {
-                Kt[(i + 0) * ldp + sl] = (uint16_t)(pk.x & 0xFFFFu); Kt[(i + 1) * ldp + sl] = (uint16_t)(pk.x >> 16);
-                Kt[(i + 2) * ldp + sl] = (uint16_t)(pk.y & 0xFFFFu); Kt[(i + 3) * ldp + sl] = (uint16_t)(pk.y >> 16);
-                Kt[(i + 4) * ldp + sl] = (uint16_t)(pk.z & 0xFFFFu); Kt[(i + 5) * ldp + sl] = (uint16_t)(pk.z >> 16);
-                Kt[(i + 6) * ldp + sl] = (uint16_t)(pk.w & 0xFFFFu); Kt[(i + 7) * ldp + sl] = (uint16_t)(pk.w >> 16);
+        look_up(v0 + LM_KT, buf ^ 1);
+        // four independent 16-byte loads in flight per thread, then their stores
+        for (int base = 0; base < nkl; base += 4 * LM_NT) {
+            u32x4 pk[4];
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int idx = base + c * LM_NT + tid;
+                pk[c] = (u32x4){0u, 0u, 0u, 0u};
+                if (idx < nkl) {
+                    const int sl = idx / (d / 8), i = (idx - sl * (d / 8)) * 8;
+                    const char* src = rowp[buf][sl].k;
+                    if (src) pk[c] = *(const u32x4*)((const uint16_t*)src + i);
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const int idx = base + c * LM_NT + tid;
+                if (idx < nkl) {
+                    const int sl = idx / (d / 8), i = (idx - sl * (d / 8)) * 8;
+                    *(u32x4*)&Ks[sl * ldq + i] = pk[c];
+                    if (!WIDE && !ownv && i < e) transposed(pk[c], i, sl);
+                }
             }
         }
         if (!WIDE && ownv)
-            for (int idx = tid; idx < LM_KT * (e / 8); idx += LM_NT) {
-                const int sl = idx / (e / 8), i = (idx - sl * (e / 8)) * 8;
-                const int v = v0 + sl;
-                u32x4 pk = {0u, 0u, 0u, 0u};
-                if (v < total) pk = *(const u32x4*)((const uint16_t*)la_row<2>(a, sg, g, v, sink_hi, main_lo, pool).v + i);
-                Kt[(i + 0) * ldp + sl] = (uint16_t)(pk.x & 0xFFFFu); Kt[(i + 1) * ldp + sl] = (uint16_t)(pk.x >> 16);
-                Kt[(i + 2) * ldp + sl] = (uint16_t)(pk.y & 0xFFFFu); Kt[(i + 3) * ldp + sl] = (uint16_t)(pk.y >> 16);
-                Kt[(i + 4) * ldp + sl] = (uint16_t)(pk.z & 0xFFFFu); Kt[(i + 5) * ldp + sl] = (uint16_t)(pk.z >> 16);
-                Kt[(i + 6) * ldp + sl] = (uint16_t)(pk.w & 0xFFFFu); Kt[(i + 7) * ldp + sl] = (uint16_t)(pk.w >> 16);
+            for (int base = 0; base < nvl; base += 4 * LM_NT) {
+                u32x4 pk[4];
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const int idx = base + c * LM_NT + tid;
+                    pk[c] = (u32x4){0u, 0u, 0u, 0u};
+                    if (idx < nvl) {
+                        const int sl = idx / (e / 8), i = (idx - sl * (e / 8)) * 8;
+                        const char* src = rowp[buf][sl].v;
+                        if (src) pk[c] = *(const u32x4*)((const uint16_t*)src + i);
+                    }
+                }
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    const int idx = base + c * LM_NT + tid;
+                    if (idx < nvl) { const int sl = idx / (e / 8), i = (idx - sl * (e / 8)) * 8; transposed(pk[c], i, sl); }
+                }
             }
         __syncthreads();
         f32x4 S[4];
