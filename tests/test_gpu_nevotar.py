@@ -546,3 +546,44 @@ def test_drawn_models_whole_in_portions_and_decoded_in_both_formats(tmp_path, se
             assert at == 170 and err(np.concatenate(out), want) < tol, (dtype, "portions")
         finally:
             m.close()
+
+
+def test_a_trace_of_mixed_steps_replayed_by_the_command_line_runner(tmp_path):
+    """bin/trace_run on a small model: five requests over four slots and a pool of 7 pages (their sum: 9), portions beside single tokens,
+    requests that end and whose pages and slots the next ones take."""
+    import json
+    import os
+    import subprocess
+    import sys
+    cfg = U.small_config()
+    P = U.random_weights(cfg, 19)
+    ckpt = U.write_checkpoint(str(tmp_path / "ckpt"), cfg, P)
+    reqs = {n: U.tokens(k, cfg["vocab"], 80 + i) for i, (n, k) in enumerate((("a", 90), ("b", 7), ("c", 130), ("d", 40), ("e", 66)))}
+    want = {n: O.forward(cfg, P, t) for n, t in reqs.items()}
+    plan = [[("a", 50), ("b", 2)], [("a", 1), ("b", 1), ("c", 64)], [("c", 2), ("a", 39), ("b", 4), ("d", 30)], [("d", 10), ("c", 60)],
+            [("e", 3)], [("e", 62), ("c", 0)], [("e", 1)]]
+    at = {n: 0 for n in reqs}
+    lines, asked = [], []
+    for n_step, step in enumerate(plan):
+        entries, end, rows = [], [], []
+        for n, c in step:
+            c = c or len(reqs[n]) - at[n]
+            wanted = sorted({0, c - 1, c // 2})
+            entries.append(dict(id=n, tokens=reqs[n][at[n]:at[n] + c], want=wanted))
+            rows += [(n, at[n] + k) for k in wanted]
+            at[n] += c
+            if at[n] == len(reqs[n]):
+                end.append(n)
+        lines.append(json.dumps(dict(step=n_step, entries=entries, end=end)))
+        asked.append(rows)
+    assert all(at[n] == len(reqs[n]) for n in reqs)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for dtype, tol, err in (("float32", TOL_F32, _err), ("bfloat16", TOL_BF16, _err_long)):       # (few rows, drawn from five requests)
+        out = tmp_path / ("out_" + dtype)
+        run = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", ckpt, "--dtype", dtype, "--out", str(out), "--max-tokens", "448"],
+                             input="\n".join(lines) + "\n", capture_output=True, text=True, timeout=600)
+        assert run.returncode == 0, run.stderr[-2000:]
+        assert [x for x in run.stdout.split("\n") if x.startswith("done")] == ["done %d" % i for i in range(len(plan))]
+        got = np.concatenate([np.fromfile(out / ("%d.f32" % i), "<f4").reshape(-1, cfg["vocab"]) for i in range(len(plan))])
+        ref = np.stack([want[n][p] for rows in asked for n, p in rows])
+        assert got.shape == ref.shape and err(got, ref) < tol, dtype
