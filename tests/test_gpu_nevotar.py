@@ -472,8 +472,15 @@ def test_a_step_larger_than_one_pass_is_cut_into_passes(tmp_path):
         m.close()
 
 
-def test_matrix_core_attention_of_prompt_passes_against_the_plain_kernel(tmp_path):
-    cfg = _wide_config()
+def _many_heads_config(heads, kv_heads):
+    """Mixed heads in numbers other than a power of two, at sizes the matrix-core kernel takes."""
+    return U.config([_par(U.left(heads=heads, kv_heads=kv_heads, dim=32, vdim=32, size=70, dims=16, scale=0.2), U.right(heads=4, vdim=32, state=32, groups=2, conv=4, norm_groups=2),
+                          None)], vocab=256, width=128, groups=2)
+
+
+@pytest.mark.parametrize("cfg", [_wide_config(), _many_heads_config(12, 4), _many_heads_config(6, 3), _many_heads_config(9, 1)],
+                         ids=["four heads", "twelve heads", "six heads", "nine heads"])
+def test_matrix_core_attention_of_prompt_passes_against_the_plain_kernel(tmp_path, cfg):
     P = U.random_weights(cfg, 17)
     toks = U.tokens(300, cfg["vocab"], 17)
     want = O.forward(cfg, P, toks)
