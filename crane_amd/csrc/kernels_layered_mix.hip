@@ -371,21 +371,22 @@ __global__ __launch_bounds__(64) void lay_attn_talk_merge_kernel(LAttnArgs a, in
 // barrier it mixes the H raw scores of each of its (position, key) places with its line of the matrix in the accumulator's own
 // layout (A[i = lane % 16][k = 4 (lane / 16) ..], B[k][j = lane % 16], D[i = 4 (lane / 16) + r][j = lane % 16]); mask, running
 // max / sum and the weights are f32, the weights enter P V as a bf16 hi + lo pair (two products per tile).
-constexpr int LTM_KT = 64, LTM_LDS = 68;          // keys per tile; f32 stride of a raw-score row (68: the two half-waves of a read hit disjoint banks)
-static size_t lay_talk_mfma_lds(int H, int G, int d, int e) {
-    return (size_t)(G * LTM_KT * (d + 8) + G * e * (LTM_KT + 8) + 2 * H * 16 * (LTM_KT + 8)) * sizeof(uint16_t) +
-           (size_t)(H * 16 * LTM_LDS + H * H) * sizeof(float);
+// KT keys per tile (64, or 32 where that is what fits in LDS: more heads); a raw-score row holds KT + 4 floats, so that the two half-waves
+// of a read hit disjoint banks
+static size_t lay_talk_mfma_lds(int H, int G, int d, int e, int KT) {
+    return (size_t)(G * KT * (d + 8) + G * e * (KT + 8) + 2 * H * 16 * (KT + 8)) * sizeof(uint16_t) + (size_t)(H * 16 * (KT + 4) + H * H) * sizeof(float);
 }
-template <int NDMAX, int NEMAX, int NT>
+template <int NDMAX, int NEMAX, int NT, int KT>
 __global__ __launch_bounds__(NT) void lay_attn_talk_mfma_kernel(LAttnArgs a, const float* __restrict__ talk) {
+    constexpr int LTM_KT = KT, LTM_LDS = KT + 4, NS = KT / 16;      // sub-tiles of 16 keys
     extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
     const int d = a.d, e = a.e, H = a.H, G = a.G, nrep = H / G;
     const int ldq = d + 8, ldp = LTM_KT + 8;
-    uint16_t* Ks = smem;                               // [G][64][d + 8]
-    uint16_t* Vt = Ks + G * LTM_KT * ldq;              // [G][e][72] the value tiles transposed (the B operand of P V: 4 keys of one element)
-    uint16_t* Ph = Vt + G * e * ldp;                   // [H][16][72] hi
+    uint16_t* Ks = smem;                               // [G][KT][d + 8]
+    uint16_t* Vt = Ks + G * LTM_KT * ldq;              // [G][e][KT + 8] the value tiles transposed (the B operand of P V: 4 keys of one element)
+    uint16_t* Ph = Vt + G * e * ldp;                   // [H][16][KT + 8] hi
     uint16_t* Pl = Ph + H * 16 * ldp;                  // ... lo
-    float* Sr = (float*)(Pl + H * 16 * ldp);           // [H][16][68] raw scores of every head
+    float* Sr = (float*)(Pl + H * 16 * ldp);           // [H][16][KT + 4] raw scores of every head
     float* tk = Sr + H * 16 * LTM_LDS;                 // [H][H]
     const LaySegDev sg = a.segs[blockIdx.x];
     const int p0 = (int)blockIdx.y * 16;
@@ -479,41 +480,41 @@ __global__ __launch_bounds__(NT) void lay_attn_talk_mfma_kernel(LAttnArgs a, con
             }
         }
         __syncthreads();
-        f32x4 S[4];
+        f32x4 S[NS];
 #pragma unroll
-        for (int t = 0; t < 4; ++t) S[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        for (int t = 0; t < NS; ++t) S[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int kk = 0; kk < NDMAX; ++kk) {
             if (kk < nd) {
                 const bf16x4 qa = qf[kk];
 #pragma unroll
-                for (int t = 0; t < 4; ++t) {
+                for (int t = 0; t < NS; ++t) {
                     const bf16x4 kb = *(const bf16x4*)&kg[(t * 16 + lr) * ldq + kk * 16 + 4 * lg];
                     S[t] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(qa, kb, S[t], 0, 0, 0);
                 }
             }
         }
 #pragma unroll
-        for (int t = 0; t < 4; ++t)
+        for (int t = 0; t < NS; ++t)
 #pragma unroll
             for (int r = 0; r < 4; ++r) sr[(4 * lg + r) * LTM_LDS + t * 16 + lr] = S[t][r] * a.scale;
         __syncthreads();                   // every head's raw scores are in LDS
 #pragma unroll
-        for (int t = 0; t < 4; ++t) S[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        for (int t = 0; t < NS; ++t) S[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
         for (int g2 = 0; g2 < H; ++g2) {
             const float w = tk[h * H + g2];
             const float* so = Sr + (size_t)g2 * 16 * LTM_LDS;
 #pragma unroll
-            for (int t = 0; t < 4; ++t)
+            for (int t = 0; t < NS; ++t)
 #pragma unroll
                 for (int r = 0; r < 4; ++r) S[t][r] = fmaf(w, so[(4 * lg + r) * LTM_LDS + t * 16 + lr], S[t][r]);
         }
         float corr[4];
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            float sc[4], tmax = -INFINITY;
+            float sc[NS], tmax = -INFINITY;
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
+            for (int t = 0; t < NS; ++t) {
                 const int v = v0 + t * 16 + lr, j = main_lo + v;
                 const bool vis = qok[r] && v < total && j <= qpos[r] && qpos[r] - j < win;
                 sc[t] = vis ? S[t][r] : -INFINITY;
@@ -524,7 +525,7 @@ __global__ __launch_bounds__(NT) void lay_attn_talk_mfma_kernel(LAttnArgs a, con
             corr[r] = mn == -INFINITY ? 1.f : __expf(m[r] - mn);
             float psum = 0.f;
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
+            for (int t = 0; t < NS; ++t) {
                 const float p = sc[t] == -INFINITY ? 0.f : __expf(sc[t] - mn);
                 psum += p;
                 const uint16_t hi = f32_to_bf16(p);
@@ -541,7 +542,7 @@ __global__ __launch_bounds__(NT) void lay_attn_talk_mfma_kernel(LAttnArgs a, con
             for (int r = 0; r < 4; ++r) O[n][r] *= corr[r];
         __syncthreads();                   // the wave's weights are in LDS
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
+        for (int ks = 0; ks < NS; ++ks) {
             const bf16x4 ah = *(const bf16x4*)&ph[lr * ldp + ks * 16 + 4 * lg];
             const bf16x4 al = *(const bf16x4*)&pl[lr * ldp + ks * 16 + 4 * lg];
 #pragma unroll
@@ -565,24 +566,30 @@ __global__ __launch_bounds__(NT) void lay_attn_talk_mfma_kernel(LAttnArgs a, con
 }
 bool lay_attn_talk_mfma_fits(int H, int G, int d, int e) {
     return H > 0 && H <= 16 && G > 0 && H % G == 0 && d > 0 && e > 0 && d % 16 == 0 && e % 16 == 0 && d <= 128 && e <= 128 &&
-           lay_talk_mfma_lds(H, G, d, e) <= LT_LDS_MAX;
+           lay_talk_mfma_lds(H, G, d, e, 32) <= LT_LDS_MAX;
 }
-template <int NT>
+template <int NT, int KT>
 static void lay_attn_talk_mfma_go(const LAttnArgs& a, const float* talk, dim3 grid, size_t lds, hipStream_t s) {
     static bool raised = false;            // per instantiation
     if (!raised) {
-        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&lay_attn_talk_mfma_kernel<8, 8, NT>), hipFuncAttributeMaxDynamicSharedMemorySize,
+        (void)hipFuncSetAttribute(reinterpret_cast<const void*>(&lay_attn_talk_mfma_kernel<8, 8, NT, KT>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                   (int)LT_LDS_MAX);
         raised = true;
     }
-    hipLaunchKernelGGL((lay_attn_talk_mfma_kernel<8, 8, NT>), grid, dim3((unsigned)(64 * a.H)), lds, s, a, talk);
+    hipLaunchKernelGGL((lay_attn_talk_mfma_kernel<8, 8, NT, KT>), grid, dim3((unsigned)(64 * a.H)), lds, s, a, talk);
 }
 void launch_lay_attn_talk_mfma(const LAttnArgs& a, const float* talk, int nseg, int max_n, hipStream_t s) {
     if (nseg <= 0 || max_n <= 0) return;
     const dim3 grid((unsigned)nseg, (unsigned)((max_n + 15) / 16));
-    const size_t lds = lay_talk_mfma_lds(a.H, a.G, a.d, a.e);
-    if (a.H <= 8) lay_attn_talk_mfma_go<512>(a, talk, grid, lds, s);
-    else lay_attn_talk_mfma_go<1024>(a, talk, grid, lds, s);
+    const bool wide = lay_talk_mfma_lds(a.H, a.G, a.d, a.e, 64) <= LT_LDS_MAX;      // 64-key tiles where they fit
+    const size_t lds = lay_talk_mfma_lds(a.H, a.G, a.d, a.e, wide ? 64 : 32);
+    if (a.H <= 8) {
+        if (wide) lay_attn_talk_mfma_go<512, 64>(a, talk, grid, lds, s);
+        else lay_attn_talk_mfma_go<512, 32>(a, talk, grid, lds, s);
+    } else {
+        if (wide) lay_attn_talk_mfma_go<1024, 64>(a, talk, grid, lds, s);
+        else lay_attn_talk_mfma_go<1024, 32>(a, talk, grid, lds, s);
+    }
 }
 
 template <int KVT, int RPG, int NACC>

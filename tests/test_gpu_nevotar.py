@@ -478,8 +478,8 @@ def _many_heads_config(heads, kv_heads):
                           None)], vocab=256, width=128, groups=2)
 
 
-@pytest.mark.parametrize("cfg", [_wide_config(), _many_heads_config(12, 4), _many_heads_config(6, 3), _many_heads_config(9, 1)],
-                         ids=["four heads", "twelve heads", "six heads", "nine heads"])
+@pytest.mark.parametrize("cfg", [_wide_config(), _many_heads_config(12, 4), _many_heads_config(6, 3), _many_heads_config(9, 1), _many_heads_config(16, 4)],
+                         ids=["four heads", "twelve heads", "six heads", "nine heads", "sixteen heads (tiles of 32 keys)"])
 def test_matrix_core_attention_of_prompt_passes_against_the_plain_kernel(tmp_path, cfg):
     P = U.random_weights(cfg, 17)
     toks = U.tokens(300, cfg["vocab"], 17)
