@@ -373,18 +373,21 @@ __global__ __launch_bounds__(64) void lay_attn_talk_merge_kernel(LAttnArgs a, in
 // max / sum and the weights are f32, the weights enter P V as a bf16 hi + lo pair (two products per tile).
 // KT keys per tile (64, or 32 where that is what fits in LDS: more heads); a raw-score row holds KT + 4 floats, so that the two half-waves
 // of a read hit disjoint banks
-static size_t lay_talk_mfma_lds(int H, int G, int d, int e, int KT) {
-    return (size_t)(G * KT * (d + 8) + G * e * (KT + 8) + 2 * H * 16 * (KT + 8)) * sizeof(uint16_t) + (size_t)(H * 16 * (KT + 4) + H * H) * sizeof(float);
+// Gv value heads (consecutive key heads may share one); mixed: the raw-score rows and the matrix are needed
+static size_t lay_talk_mfma_lds(int H, int G, int Gv, int d, int e, int KT, bool mixed) {
+    return (size_t)(G * KT * (d + 8) + Gv * e * (KT + 8) + 2 * H * 16 * (KT + 8)) * sizeof(uint16_t) +
+           (mixed ? (size_t)(H * 16 * (KT + 4) + H * H) * sizeof(float) : 0);
 }
 template <int NDMAX, int NEMAX, int NT, int KT>
 __global__ __launch_bounds__(NT) void lay_attn_talk_mfma_kernel(LAttnArgs a, const float* __restrict__ talk) {
     constexpr int LTM_KT = KT, LTM_LDS = KT + 4, NS = KT / 16;      // sub-tiles of 16 keys
     extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
-    const int d = a.d, e = a.e, H = a.H, G = a.G, nrep = H / G;
+    const int d = a.d, e = a.e, H = a.H, G = a.G, nrep = H / G, vdiv = max(a.v_div, 1), Gv = G / vdiv;
     const int ldq = d + 8, ldp = LTM_KT + 8;
+    const bool mixed = talk != nullptr;                // null: every head keeps its own scores (the kernel then is plain attention, one wave per head)
     uint16_t* Ks = smem;                               // [G][KT][d + 8]
-    uint16_t* Vt = Ks + G * LTM_KT * ldq;              // [G][e][KT + 8] the value tiles transposed (the B operand of P V: 4 keys of one element)
-    uint16_t* Ph = Vt + G * e * ldp;                   // [H][16][KT + 8] hi
+    uint16_t* Vt = Ks + G * LTM_KT * ldq;              // [Gv][e][KT + 8] the value tiles transposed (the B operand of P V: 4 keys of one element)
+    uint16_t* Ph = Vt + Gv * e * ldp;                  // [H][16][KT + 8] hi
     uint16_t* Pl = Ph + H * 16 * ldp;                  // ... lo
     float* Sr = (float*)(Pl + H * 16 * ldp);           // [H][16][KT + 4] raw scores of every head
     float* tk = Sr + H * 16 * LTM_LDS;                 // [H][H]
@@ -395,7 +398,7 @@ __global__ __launch_bounds__(NT) void lay_attn_talk_mfma_kernel(LAttnArgs a, con
     const int tid = threadIdx.x, nt = 64 * H, lane = tid & 63, h = tid >> 6, lr = lane & 15, lg = lane >> 4;
     const int g = h / nrep;
     const int win = (int)min(a.win, 1ll << 30);
-    for (int idx = tid; idx < H * H; idx += nt) tk[idx] = talk[idx];
+    if (mixed) for (int idx = tid; idx < H * H; idx += nt) tk[idx] = talk[idx];
     // this lane's part of the q fragments: position p0 + lr, elements kk 16 + 4 lg .. + 3 of head h
     const int nd = d / 16, ne = e / 16;
     bf16x4 qf[NDMAX];
@@ -421,19 +424,18 @@ __global__ __launch_bounds__(NT) void lay_attn_talk_mfma_kernel(LAttnArgs a, con
     uint16_t* ph = Ph + h * 16 * ldp;
     uint16_t* pl = Pl + h * 16 * ldp;
     const uint16_t* kg = Ks + g * LTM_KT * ldq;
-    const uint16_t* vg = Vt + g * e * ldp;
+    const uint16_t* vg = Vt + (g / vdiv) * e * ldp;
     float* sr = Sr + h * 16 * LTM_LDS;
-    // the cached row of every key of a tile (key head 0; -1 past the end), looked up one tile ahead so that the tile's loads do not
-    // wait for the page table
+    // the page of every key of a tile (-1 past the end), looked up one tile ahead so that the tile's loads do not wait for the page table
     __shared__ int rowb[2][LTM_KT];
     auto look_up = [&](int v0, int buf) {
         if (tid < LTM_KT) {
             const int v = v0 + tid, j = main_lo + v;
-            rowb[buf][tid] = v < total ? a.bt[sg.bt_off + j / a.page] * G * a.page + j % a.page : -1;
+            rowb[buf][tid] = v < total ? a.bt[sg.bt_off + j / a.page] : -1;
         }
     };
     look_up(0, 0);
-    const int nk = G * LTM_KT * (d / 8), nv = G * LTM_KT * (e / 8);
+    const int nk = G * LTM_KT * (d / 8), nv = Gv * LTM_KT * (e / 8);
     for (int v0 = 0, buf = 0; v0 < total; v0 += LTM_KT, buf ^= 1) {
         __syncthreads();                   // the previous tile is consumed: keys, values and raw scores may be replaced
         look_up(v0 + LTM_KT, buf ^ 1);
@@ -445,8 +447,8 @@ __global__ __launch_bounds__(NT) void lay_attn_talk_mfma_kernel(LAttnArgs a, con
                 const int idx = base + c * nt + tid;
                 pk[c] = (u32x4){0u, 0u, 0u, 0u};
                 if (idx < nk) {
-                    const int rw = idx / (d / 8), i = (idx - rw * (d / 8)) * 8, kgi = rw / LTM_KT, rb = rowb[buf][rw - kgi * LTM_KT];
-                    if (rb >= 0) pk[c] = *(const u32x4*)((const uint16_t*)a.kpool + ((size_t)rb + (size_t)kgi * a.page) * d + i);
+                    const int rw = idx / (d / 8), i = (idx - rw * (d / 8)) * 8, kgi = rw / LTM_KT, sl = rw - kgi * LTM_KT, pg = rowb[buf][sl];
+                    if (pg >= 0) pk[c] = *(const u32x4*)((const uint16_t*)a.kpool + (((size_t)pg * G + kgi) * a.page + (size_t)((main_lo + v0 + sl) % a.page)) * d + i);
                 }
             }
 #pragma unroll
@@ -462,8 +464,8 @@ __global__ __launch_bounds__(NT) void lay_attn_talk_mfma_kernel(LAttnArgs a, con
                 const int idx = base + c * nt + tid;
                 pk[c] = (u32x4){0u, 0u, 0u, 0u};
                 if (idx < nv) {
-                    const int rw = idx / (e / 8), i = (idx - rw * (e / 8)) * 8, kgi = rw / LTM_KT, rb = rowb[buf][rw - kgi * LTM_KT];
-                    if (rb >= 0) pk[c] = *(const u32x4*)((const uint16_t*)a.vpool + ((size_t)rb + (size_t)kgi * a.page) * e + i);
+                    const int rw = idx / (e / 8), i = (idx - rw * (e / 8)) * 8, kgi = rw / LTM_KT, sl = rw - kgi * LTM_KT, pg = rowb[buf][sl];
+                    if (pg >= 0) pk[c] = *(const u32x4*)((const uint16_t*)a.vpool + (((size_t)pg * Gv + kgi) * a.page + (size_t)((main_lo + v0 + sl) % a.page)) * e + i);
                 }
             }
 #pragma unroll
@@ -494,20 +496,27 @@ __global__ __launch_bounds__(NT) void lay_attn_talk_mfma_kernel(LAttnArgs a, con
                 }
             }
         }
-#pragma unroll
-        for (int t = 0; t < NS; ++t)
-#pragma unroll
-            for (int r = 0; r < 4; ++r) sr[(4 * lg + r) * LTM_LDS + t * 16 + lr] = S[t][r] * a.scale;
-        __syncthreads();                   // every head's raw scores are in LDS
-#pragma unroll
-        for (int t = 0; t < NS; ++t) S[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
-        for (int g2 = 0; g2 < H; ++g2) {
-            const float w = tk[h * H + g2];
-            const float* so = Sr + (size_t)g2 * 16 * LTM_LDS;
+        if (mixed) {
 #pragma unroll
             for (int t = 0; t < NS; ++t)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) S[t][r] = fmaf(w, so[(4 * lg + r) * LTM_LDS + t * 16 + lr], S[t][r]);
+                for (int r = 0; r < 4; ++r) sr[(4 * lg + r) * LTM_LDS + t * 16 + lr] = S[t][r] * a.scale;
+            __syncthreads();               // every head's raw scores are in LDS
+#pragma unroll
+            for (int t = 0; t < NS; ++t) S[t] = (f32x4){0.f, 0.f, 0.f, 0.f};
+            for (int g2 = 0; g2 < H; ++g2) {
+                const float w = tk[h * H + g2];
+                const float* so = Sr + (size_t)g2 * 16 * LTM_LDS;
+#pragma unroll
+                for (int t = 0; t < NS; ++t)
+#pragma unroll
+                    for (int r = 0; r < 4; ++r) S[t][r] = fmaf(w, so[(4 * lg + r) * LTM_LDS + t * 16 + lr], S[t][r]);
+            }
+        } else {
+#pragma unroll
+            for (int t = 0; t < NS; ++t)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) S[t][r] *= a.scale;
         }
         float corr[4];
 #pragma unroll
@@ -564,9 +573,9 @@ __global__ __launch_bounds__(NT) void lay_attn_talk_mfma_kernel(LAttnArgs a, con
             if (n < ne) a.out[(size_t)(sg.row0 + p0 + 4 * lg + r) * a.ldo + h * e + n * 16 + lr] = O[n][r] * inv;
     }
 }
-bool lay_attn_talk_mfma_fits(int H, int G, int d, int e) {
-    return H > 0 && H <= 16 && G > 0 && H % G == 0 && d > 0 && e > 0 && d % 16 == 0 && e % 16 == 0 && d <= 128 && e <= 128 &&
-           lay_talk_mfma_lds(H, G, d, e, 32) <= LT_LDS_MAX;
+bool lay_attn_talk_mfma_fits(int H, int G, int d, int e, int v_div, bool mixed) {
+    return H > 0 && H <= 16 && G > 0 && H % G == 0 && v_div > 0 && G % v_div == 0 && d > 0 && e > 0 && d % 16 == 0 && e % 16 == 0 && d <= 128 &&
+           e <= 128 && lay_talk_mfma_lds(H, G, G / v_div, d, e, 32, mixed) <= LT_LDS_MAX;
 }
 template <int NT, int KT>
 static void lay_attn_talk_mfma_go(const LAttnArgs& a, const float* talk, dim3 grid, size_t lds, hipStream_t s) {
@@ -581,8 +590,9 @@ static void lay_attn_talk_mfma_go(const LAttnArgs& a, const float* talk, dim3 gr
 void launch_lay_attn_talk_mfma(const LAttnArgs& a, const float* talk, int nseg, int max_n, hipStream_t s) {
     if (nseg <= 0 || max_n <= 0) return;
     const dim3 grid((unsigned)nseg, (unsigned)((max_n + 15) / 16));
-    const bool wide = lay_talk_mfma_lds(a.H, a.G, a.d, a.e, 64) <= LT_LDS_MAX;      // 64-key tiles where they fit
-    const size_t lds = lay_talk_mfma_lds(a.H, a.G, a.d, a.e, wide ? 64 : 32);
+    const int Gv = a.G / std::max(a.v_div, 1);
+    const bool wide = lay_talk_mfma_lds(a.H, a.G, Gv, a.d, a.e, 64, talk != nullptr) <= LT_LDS_MAX;      // 64-key tiles where they fit
+    const size_t lds = lay_talk_mfma_lds(a.H, a.G, Gv, a.d, a.e, wide ? 64 : 32, talk != nullptr);
     if (a.H <= 8) {
         if (wide) lay_attn_talk_mfma_go<512, 64>(a, talk, grid, lds, s);
         else lay_attn_talk_mfma_go<512, 32>(a, talk, grid, lds, s);

@@ -325,9 +325,10 @@ void launch_lay_ssm_out(const float* o, const float* x, int ldx, int x_off, cons
 void launch_lay_attn_talk(const LAttnArgs& a, const float* talk, int nseg, int max_n, int kvt, hipStream_t s);
 bool lay_attn_talk_fits(int H, int G, int d, int e);
 // bf16 key / value pages, up to 16 heads, d and e multiples of 16 up to 128: the matrix-core form for prompt passes (16 positions a block,
-// one wave per head)
+// one wave per head).  talk null: no mixing -- plain attention in this blocking (all heads of a position share the staged key and
+// value tiles), which also takes LAttnArgs::v_div
 void launch_lay_attn_talk_mfma(const LAttnArgs& a, const float* talk, int nseg, int max_n, hipStream_t s);
-bool lay_attn_talk_mfma_fits(int H, int G, int d, int e);
+bool lay_attn_talk_mfma_fits(int H, int G, int d, int e, int v_div = 1, bool mixed = true);
 
 // router: z = h . Wr^T in f32 over E outputs, scores by rs (sigmoid of each / softmax over all), the `top` largest choice scores
 // (score + correction, inside the best groups; lowest index first among equals) -> sel [T top], wsel [T slots] = their scores

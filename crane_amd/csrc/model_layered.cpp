@@ -1543,9 +1543,22 @@ void Model::step_batch(const StepItem* items, size_t n_items, float* logits_out,
                     ex.Gv = G; ex.qt_coef = sp.qt_coef; ex.qt_every = (int)sp.qt_every;
                     launch_lay_qk_prep(L.P, w.in_rows, w.q_off, w.k_off, w.v_off, 2 * H, 2 * G, d, e, nullptr, nullptr, cfg.eps, 0, false, nullptr, 1.f,
                                        kv_pool + w.k_pool_off, kv_pool + w.v_pool_off, kv_mode, d_bt, d_segs, d_rowseg, T, page, s, 0, 0, nullptr, nullptr, &ex);
-                    LayerSpec two = sp;
-                    two.heads = 2 * H; two.kv_heads = 2 * G;
-                    run_attention(two, w, L.P, w.in_rows, w.q_off, 0, d, e, nullptr, 0, 1.f, 2);
+                    if (L.attn_mfma && kv_mode == KV_BF16 && !all_decode && max_n >= 16 && lay_attn_talk_mfma_fits(2 * H, 2 * G, d, e, 2, false) &&
+                        w.in_rows % 4 == 0 && w.q_off % 4 == 0) {
+                        // prompt passes: a block of 16 positions with one wave per (head, map), all of them on the same staged tiles
+                        LAttnArgs a;
+                        a.proj = L.P; a.ldp = w.in_rows; a.q_off = w.q_off; a.g_off = 0;
+                        a.out = L.O; a.ldo = 2 * H * e; a.out_scale = 1.f;
+                        a.kpool = kv_pool + w.k_pool_off; a.vpool = kv_pool + w.v_pool_off; a.bt = d_bt; a.segs = d_segs;
+                        a.tiles = nullptr; a.ntiles = 0; a.r1 = a.r2 = nullptr;
+                        a.H = 2 * H; a.G = 2 * G; a.d = d; a.e = e; a.page = page; a.scale = sp.scale; a.win = sp.win; a.keep = 0;
+                        a.bias = LBIAS_NONE; a.gate = LGATE_NONE; a.v_div = 2;
+                        launch_lay_attn_talk_mfma(a, nullptr, nseg, max_n, s);
+                    } else {
+                        LayerSpec two = sp;
+                        two.heads = 2 * H; two.kv_heads = 2 * G;
+                        run_attention(two, w, L.P, w.in_rows, w.q_off, 0, d, e, nullptr, 0, 1.f, 2);
+                    }
                     launch_lay_diff_combine(L.O, L.O2, T, H, G, e, w.lambda, 1.f - sp.diff, cfg.eps, s);
                     oa = L.O2; on = H * e;
                 } else if (sp.mixer == LMIX_HGRN) {
